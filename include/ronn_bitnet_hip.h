@@ -1,0 +1,207 @@
+/*
+ * ronn_bitnet_hip.h - C ABI of the MI355X (gfx950) BitNet ternary hot path.
+ *
+ * This is the boundary a host-language binding (the Rust `ronn-providers` crate
+ * through an `extern "C"` block, or ctypes, or C++) calls.  Plain pointers and
+ * sizes only.  Citations name the reference code each entry point stands in for,
+ * relative to the reference checkout's crates/ronn-providers/src/bitnet/.
+ *
+ * Conventions
+ *   - Every function returns RBN_OK (0) or a negative rbn_status.  Nothing throws
+ *     or aborts across this boundary.  rbn_last_error() returns the message of the
+ *     calling thread's most recent failure.
+ *   - Pointers named d_* are device pointers (from rbn_malloc, or any hipMalloc'd
+ *     memory of the same device); h_* are host pointers.  All are caller-owned.
+ *   - A context owns one HIP stream of default priority.  Calls on one context are
+ *     serialised by an internal lock, so a context may be shared by threads
+ *     (the reference's CompiledKernel is Send + Sync, ronn-core types.rs:153).
+ *     Compute calls are asynchronous on that stream unless they return a value
+ *     through a host pointer; rbn_sync() waits for the stream.
+ *   - Matrices are row-major.  A is activations [M,K], B is weights [K,N], the
+ *     result is [M,N] (kernels.rs:134-178).
+ *
+ * Weight formats
+ *   "packed"  The reference's TernaryTensor.packed_data (quantization.rs:131-153,
+ *             249-260): element i of the flattened tensor is the 2-bit field at bit
+ *             2*(i%4) of byte i/4; 00 = -1, 01 = 0, 10 = +1, 11 never produced and
+ *             read as 0 (quantization.rs:285-290).  ceil(n/4) bytes; device buffers
+ *             must have rbn_packed_capacity(n) bytes.
+ *   "tiled"   Device-internal layout the matmul kernels stream: u32 word
+ *             [kb][n], kb in [0,Kpad/16), n in [0,Npad), holds the 16 weights
+ *             k = 16*kb + 4*s + b of column n as the 2-bit field at bit 8*b + 2*s
+ *             (so (word >> 2*s) & 0x03030303 is four int8-ready codes of four
+ *             consecutive k).  Code = value + 1 (same as "packed"); 11 and padding
+ *             are stored as 01 (zero).  Kpad = K rounded up to 64, Npad = N rounded
+ *             up to 64.  Built from "packed" by rbn_tile_weights().
+ */
+#ifndef RONN_BITNET_HIP_H
+#define RONN_BITNET_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct rbn_ctx rbn_ctx;
+
+typedef enum rbn_status {
+    RBN_OK = 0,
+    RBN_ERR_INVALID = -1,     /* bad argument (null pointer, zero/odd dimension, ...) */
+    RBN_ERR_HIP = -2,         /* a HIP runtime call failed; message has the HIP error */
+    RBN_ERR_OOM = -3,         /* device allocation failed */
+    RBN_ERR_UNSUPPORTED = -4, /* shape or mode outside what the kernels cover */
+    RBN_ERR_NO_DEVICE = -5    /* no gfx950 device visible / wrong architecture */
+} rbn_status;
+
+/* How the order-sensitive f32 sums of quantize_ternary are evaluated. */
+typedef enum rbn_sum_mode {
+    /* Bit-exact emulation of the reference's sequential f32 left fold
+     * (`iter().sum::<f32>()`, quantization.rs:79 and :96). */
+    RBN_SUM_STRICT_SEQ = 0,
+    /* Deterministic f64 tree reduction: faster and more accurate, NOT
+     * reference-exact on large tensors (threshold and scale differ). */
+    RBN_SUM_TREE = 1
+} rbn_sum_mode;
+
+typedef struct rbn_device_info {
+    char name[128];
+    char arch[64];
+    int compute_units;
+    int clock_khz;          /* max engine clock */
+    int mem_clock_khz;
+    int mem_bus_bits;
+    uint64_t hbm_bytes;
+    uint64_t l2_bytes;
+} rbn_device_info;
+
+/* ---- library / context --------------------------------------------------- */
+const char *rbn_version(void);
+/* Message of the calling thread's last failed call ("" if none). */
+const char *rbn_last_error(void);
+/* Number of HIP devices visible (0 if none or HIP cannot initialise). */
+int rbn_device_count(void);
+/* Creates a context on `device`.  Replaces BitNetExecutionProvider::with_config's
+ * resource set-up (provider.rs:77-114). */
+int rbn_ctx_create(int device, rbn_ctx **out);
+int rbn_ctx_destroy(rbn_ctx *ctx);
+int rbn_get_device_info(rbn_ctx *ctx, rbn_device_info *out);
+
+/* ---- device buffers (replaces BitNetMemoryAllocator::allocate/deallocate,
+ *      allocator.rs:99-140, with device memory instead of SystemRAM) ------- */
+int rbn_malloc(rbn_ctx *ctx, size_t bytes, void **d_out);
+int rbn_free(rbn_ctx *ctx, void *d_ptr);
+int rbn_h2d(rbn_ctx *ctx, void *d_dst, const void *h_src, size_t bytes);
+int rbn_d2h(rbn_ctx *ctx, void *h_dst, const void *d_src, size_t bytes);
+int rbn_d2d(rbn_ctx *ctx, void *d_dst, const void *d_src, size_t bytes);
+int rbn_fill_u8(rbn_ctx *ctx, void *d_dst, int value, size_t bytes);
+int rbn_sync(rbn_ctx *ctx);
+/* Bytes currently / at most allocated through rbn_malloc on this context
+ * (MemoryInfo, allocator.rs:142-148). */
+int rbn_memory_info(rbn_ctx *ctx, uint64_t *allocated, uint64_t *peak);
+
+/* Size rules of the reference allocator (allocator.rs:39-75): bytes for a tensor
+ * of `element_count` elements; dtype: 0=F32 1=F16 2=BF16 6=U8 (2-bit ternary)
+ * 8=Bool (1-bit).  Returns -1 for other dtypes. */
+int64_t rbn_tensor_bytes(uint64_t element_count, int dtype);
+size_t rbn_tensor_alignment(int dtype);
+/* Device capacity, in bytes, a "packed" buffer of n elements must have
+ * (ceil(n/4) rounded up to 16). */
+size_t rbn_packed_capacity(uint64_t n);
+/* Bytes of the "tiled" layout of a [K,N] weight matrix. */
+size_t rbn_tiled_bytes(uint64_t K, uint64_t N);
+/* Row pitch, in bytes, of quantised activations for inner dimension K (K rounded up to 64). */
+size_t rbn_act_pitch(uint64_t K);
+
+/* ---- timing on the context's stream -------------------------------------- */
+/* Records a start event on the stream.  rbn_timer_stop records the stop event,
+ * waits for it and returns the elapsed milliseconds between the two. */
+int rbn_timer_start(rbn_ctx *ctx);
+int rbn_timer_stop(rbn_ctx *ctx, float *h_ms);
+
+/* ---- (1) ternarize + pack: BitNetQuantizer::quantize_ternary,
+ *      quantization.rs:67-109, and pack_ternary_bits, :131-153 -------------- */
+/* sum_i |x_i| in f32, as the reference's fold evaluates it (mode STRICT_SEQ) or
+ * as an f64 tree rounded once to f32 (mode TREE).  With use_mask != 0 only
+ * elements with |x_i| > mask_threshold are summed (the survivors of
+ * quantization.rs:82-91) and *h_count receives how many there were; otherwise
+ * *h_count = n.  h_count may be NULL. */
+int rbn_abs_sum_f32(rbn_ctx *ctx, const float *d_x, uint64_t n, int mode, int use_mask,
+                    float mask_threshold, float *h_sum, uint64_t *h_count);
+/* pack_ternary_bits for a given threshold: writes the "packed" format. */
+int rbn_pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold,
+                     uint8_t *d_packed);
+/* The whole of quantize_ternary: threshold (quantization.rs:79), scale (:82-97),
+ * pack (:100).  Synchronous (returns scalars).  h_survivors may be NULL. */
+int rbn_quantize_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, int mode,
+                         uint8_t *d_packed, float *h_scale, float *h_threshold,
+                         uint64_t *h_survivors);
+/* dequantize_ternary, quantization.rs:182-207: code -> {-scale, 0, +scale}. */
+int rbn_dequantize_ternary(rbn_ctx *ctx, const uint8_t *d_packed, uint64_t n, float scale,
+                           float *d_out);
+/* TernaryTensor::get_value for every element (quantization.rs:275-291): int8 in
+ * {-1,0,+1}.  With rows/cols/pitch it writes a [rows, pitch] matrix whose columns
+ * >= cols are zero (pitch = rbn_act_pitch(cols) gives the activation format the
+ * matmuls take); rows*cols = element count.  d_rowsum (optional) gets the int32 sum
+ * of each row. */
+int rbn_unpack_ternary_i8(rbn_ctx *ctx, const uint8_t *d_packed, uint64_t rows, uint64_t cols,
+                          uint64_t pitch, int8_t *d_q, int32_t *d_rowsum);
+/* "packed" [K,N] -> "tiled" (device-internal).  No reference counterpart: the
+ * reference multiplies straight out of packed_data with get_value. */
+int rbn_tile_weights(rbn_ctx *ctx, const uint8_t *d_packed, uint64_t K, uint64_t N,
+                     uint32_t *d_tiled);
+
+/* ---- (2) activation quantisation ------------------------------------------ */
+/* Per-token absmax int8 (build-defined, no reference counterpart; the reference
+ * ternarises activations, kernels.rs:277):
+ *   g = max(max_k |x[m,k]|, 1e-5f); q = clamp(rne(x * (127/g)), -128, 127);
+ *   act_scale[m] = g / 127; rowsum[m] = sum_k q.
+ * d_q is [M, rbn_act_pitch(K)] int8 with zero padding. */
+int rbn_act_quant_i8(rbn_ctx *ctx, const float *d_x, uint64_t M, uint64_t K, int8_t *d_q,
+                     float *d_act_scale, int32_t *d_rowsum);
+/* Reference-mode activations: quantize_ternary over the whole [M,K] tensor
+ * (kernels.rs:277), expanded to int8 {-1,0,+1} in the same [M, pitch] format;
+ * act_scale[m] = the tensor's scale for every m.  Synchronous. */
+int rbn_act_quant_ternary(rbn_ctx *ctx, const float *d_x, uint64_t M, uint64_t K, int mode,
+                          int8_t *d_q, float *d_act_scale, int32_t *d_rowsum, float *h_scale,
+                          float *h_threshold);
+
+/* ---- (3)(4)(5) ternary matmul: BitNetKernel::execute_ternary_matmul,
+ *      kernels.rs:134-178, with the fused epilogue of :168 ------------------ */
+/* out[m,n] = ((float)acc[m,n] * act_scale[m]) * w_scale, acc = sum_k q[m,k]*w[k,n]
+ * in int32.  d_acc may be NULL; when given it receives the int32 accumulators.
+ * rbn_gemv_t2_i8: decode regime (M <= RBN_GEMV_MAX_M), streams the tiled weights
+ * once with int8 dot instructions.  rbn_gemm_t2_i8_mfma: prefill regime, int8 MFMA.
+ * rbn_matmul_t2_i8 picks one by M. */
+#define RBN_GEMV_MAX_M 16
+int rbn_gemv_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
+                   const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale, uint64_t M,
+                   uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);
+int rbn_gemm_t2_i8_mfma(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
+                        const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
+                        uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);
+int rbn_matmul_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
+                     const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
+                     uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);
+
+/* ---- whole execute(): CompiledKernel::execute, TernaryMatMul arm,
+ *      kernels.rs:271-283 ---------------------------------------------------- */
+/* Host f32 A [M,K] and B [K,N] in, host f32 [M,N] out; both operands ternarised
+ * per tensor on every call exactly as the reference does.  h_acc (optional) gets
+ * the int32 accumulators.  mode is an rbn_sum_mode. */
+int rbn_execute_ternary_matmul(rbn_ctx *ctx, const float *h_a, const float *h_b, uint64_t M,
+                               uint64_t N, uint64_t K, int mode, float *h_out, int32_t *h_acc);
+
+/* ---- synthetic inputs (host) ----------------------------------------------- */
+/* out[i] = (float)(sigma * z_i), z_i standard normal from a counter-based
+ * generator: two 24-bit uniforms from splitmix64(seed, i/2), Box-Muller in
+ * double.  Deterministic for (seed, i); safe to call from several threads on
+ * disjoint ranges via `first`. */
+void rbn_synth_normal_f32(uint64_t seed, double sigma, uint64_t first, uint64_t count,
+                          float *h_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RONN_BITNET_HIP_H */

@@ -1,0 +1,82 @@
+// Internal declarations shared by the translation units of libronn_bitnet_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <mutex>
+
+#include "../../include/ronn_bitnet_hip.h"
+
+struct rbn_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_start = nullptr;
+    hipEvent_t ev_stop = nullptr;
+    hipDeviceProp_t props{};
+    std::recursive_mutex lock;
+    uint64_t allocated = 0;
+    uint64_t peak = 0;
+    // Small device workspace owned by the context (reductions, sequential-sum
+    // state); grown on demand by rbn_workspace().
+    void *ws = nullptr;
+    size_t ws_bytes = 0;
+    // Pinned host mailbox for the few scalars that come back from the device.
+    void *mailbox = nullptr;
+};
+
+// Records `fmt...` as the calling thread's last error and returns `code`.
+int rbn_fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+void rbn_clear_error();
+
+// Ensures ctx->ws has at least `bytes` bytes; returns it through *out.
+int rbn_workspace(rbn_ctx *ctx, size_t bytes, void **out);
+
+#define RBN_HIP(expr)                                                                      \
+    do {                                                                                   \
+        hipError_t _e = (expr);                                                            \
+        if (_e != hipSuccess)                                                              \
+            return rbn_fail(RBN_ERR_HIP, "%s failed: %s (%s:%d)", #expr,                   \
+                            hipGetErrorString(_e), __FILE__, __LINE__);                    \
+    } while (0)
+
+#define RBN_REQUIRE(cond, ...)                                                             \
+    do {                                                                                   \
+        if (!(cond)) return rbn_fail(RBN_ERR_INVALID, __VA_ARGS__);                        \
+    } while (0)
+
+#define RBN_CHECK(expr)                                                                    \
+    do {                                                                                   \
+        int _rc = (expr);                                                                  \
+        if (_rc != RBN_OK) return _rc;                                                     \
+    } while (0)
+
+// Locks the context and makes its device current for the calling thread.
+struct CtxGuard {
+    std::unique_lock<std::recursive_mutex> lk;
+    int rc;
+    explicit CtxGuard(rbn_ctx *ctx) : lk(), rc(RBN_OK) {
+        if (!ctx) {
+            rc = rbn_fail(RBN_ERR_INVALID, "context is NULL");
+            return;
+        }
+        lk = std::unique_lock<std::recursive_mutex>(ctx->lock);
+        hipError_t e = hipSetDevice(ctx->device);
+        if (e != hipSuccess)
+            rc = rbn_fail(RBN_ERR_HIP, "hipSetDevice(%d) failed: %s", ctx->device,
+                          hipGetErrorString(e));
+    }
+};
+
+#define RBN_ENTER(ctx)      \
+    rbn_clear_error();      \
+    CtxGuard _guard(ctx);   \
+    if (_guard.rc != RBN_OK) return _guard.rc
+
+static inline uint64_t round_up_u64(uint64_t v, uint64_t m) { return (v + m - 1) / m * m; }
+
+// Layout helpers (see the header for the formats).
+static inline uint64_t rbn_kpad(uint64_t K) { return round_up_u64(K, 64); }
+static inline uint64_t rbn_npad(uint64_t N) { return round_up_u64(N, 64); }

@@ -1,0 +1,119 @@
+// Exact parallel evaluation of a sequential f32 sum of non-negative terms.
+//
+// The reference computes `data.iter().map(|x| x.abs()).sum::<f32>()`
+// (crates/ronn-providers/src/bitnet/quantization.rs:79 and :96): a strict left
+// fold S <- fl(S + x_i) in f32.  Its result depends on the order, so a tree
+// reduction cannot reproduce it.  This header holds the arithmetic that lets the
+// fold be evaluated in parallel and still bit-exactly; it is shared by the HIP
+// kernels and by a host build used in the CPU tests.
+//
+// Idea.  All terms are >= 0, so S never decreases.  While S stays inside one
+// binade [2^e, 2^(e+1)) its ulp u = 2^(e-23) is fixed: S = k*u with an integer k in
+// [2^23, 2^24).  Adding x = q*u + r (0 <= r < u) and rounding to nearest-even gives
+//      k' = k + q + [r > u/2] + [r == u/2 and (k+q) odd]
+// as long as the result stays <= 2^24 (the binade's upper edge, itself
+// representable).  So each term acts on k as  k -> k + d(k mod 2)  with two small
+// integers d(0), d(1); such maps compose associatively:
+//      (B after A)(p) = A(p) + B((p + A(p)) mod 2).
+// A block of terms therefore reduces, in parallel and in any grouping, to one pair
+// (d0,d1) that is valid for every incoming k of the assumed binade.  Values that
+// would leave the binade saturate at SEQ_SAT; the caller scans the block maps from
+// the true k, finds the first block in which k reaches 2^24, replays that one block
+// with ordinary f32 additions, and continues in the new binade.
+//
+// Subnormal S shares the ulp of the first normal binade, so biased exponent 0 is
+// treated as exponent 1 with k in [0, 2^23).
+#ifndef RONN_SEQSUM_CORE_H
+#define RONN_SEQSUM_CORE_H
+
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define SEQ_HD __host__ __device__ __forceinline__
+#else
+#define SEQ_HD inline
+#endif
+
+#define SEQ_K_LIMIT (1u << 24)  // k >= this: S has left the binade
+#define SEQ_SAT (1u << 25)      // saturation value of d0/d1
+
+struct SeqMap {
+    uint32_t d0;  // increment of k when the incoming k is even
+    uint32_t d1;  // increment of k when the incoming k is odd
+};
+
+SEQ_HD SeqMap seq_identity() {
+    SeqMap m;
+    m.d0 = 0u;
+    m.d1 = 0u;
+    return m;
+}
+
+SEQ_HD uint32_t seq_min_u32(uint32_t a, uint32_t b) { return a < b ? a : b; }
+
+// Splits the f32 state S (S >= 0, finite) into (es, k): S = k * 2^(es-150), es >= 1.
+SEQ_HD void seq_state_split(uint32_t s_bits, uint32_t *es, uint32_t *k) {
+    uint32_t e = (s_bits >> 23) & 0xffu;
+    uint32_t f = s_bits & 0x7fffffu;
+    *es = e == 0u ? 1u : e;
+    *k = e == 0u ? f : (f | 0x800000u);
+}
+
+// Inverse of seq_state_split for k < 2^24.
+SEQ_HD uint32_t seq_state_join(uint32_t es, uint32_t k) {
+    if (k < 0x800000u) return k;  // subnormal or zero; es is 1 then
+    return (es << 23) | (k & 0x7fffffu);
+}
+
+// Appends one term (|x| given as raw f32 bits with the sign bit already cleared)
+// to the running map `m`, for a state whose exponent is `es`.  A non-finite term
+// (Inf/NaN) saturates the map so the caller replays its block with real f32 adds.
+SEQ_HD SeqMap seq_append(SeqMap m, uint32_t ax_bits, uint32_t es) {
+    uint32_t e = ax_bits >> 23;
+    uint32_t f = ax_bits & 0x7fffffu;
+    uint32_t mx = e == 0u ? f : (f | 0x800000u);
+    uint32_t ex = e == 0u ? 1u : e;
+    uint32_t q, gt, eq;
+    if (e == 0xffu || ex > es) {
+        // non-finite, or a normal term at least 2 ulp-exponents above the state:
+        // the sum leaves the binade for certain.
+        q = SEQ_SAT;
+        gt = 0u;
+        eq = 0u;
+    } else {
+        uint32_t sh = es - ex;  // >= 0
+        if (sh > 31u) sh = 31u;
+        if (sh == 0u) {
+            q = mx;
+            gt = 0u;
+            eq = 0u;
+        } else {
+            uint32_t half = 1u << (sh - 1u);
+            uint32_t rem = mx & ((half << 1) - 1u);
+            q = mx >> sh;
+            gt = rem > half ? 1u : 0u;
+            eq = rem == half ? 1u : 0u;
+        }
+    }
+    uint32_t t0 = m.d0 + q;
+    uint32_t t1 = m.d1 + q;
+    // incoming parity p, current k parity = (p + d_p) & 1, after adding q: (p + t_p) & 1
+    m.d0 = seq_min_u32(t0 + gt + (eq & (t0 & 1u)), SEQ_SAT);
+    m.d1 = seq_min_u32(t1 + gt + (eq & ((t1 + 1u) & 1u)), SEQ_SAT);
+    return m;
+}
+
+// Map of "first a, then b".
+SEQ_HD SeqMap seq_compose(SeqMap a, SeqMap b) {
+    SeqMap r;
+    uint32_t b_after_even = (a.d0 & 1u) ? b.d1 : b.d0;        // parity (0 + a.d0) & 1
+    uint32_t b_after_odd = ((a.d1 + 1u) & 1u) ? b.d1 : b.d0;  // parity (1 + a.d1) & 1
+    r.d0 = seq_min_u32(a.d0 + b_after_even, SEQ_SAT);
+    r.d1 = seq_min_u32(a.d1 + b_after_odd, SEQ_SAT);
+    return r;
+}
+
+// Applies a map to a concrete k.
+SEQ_HD uint32_t seq_apply(SeqMap m, uint32_t k) { return k + ((k & 1u) ? m.d1 : m.d0); }
+
+#endif  // RONN_SEQSUM_CORE_H

@@ -1,0 +1,621 @@
+// Weight/activation ternarisation: threshold and scale sums, 2-bit packing,
+// dequantisation, expansion to int8 and the device-internal weight tiling.
+//
+// Reference: BitNetQuantizer::quantize_ternary (quantization.rs:67-109),
+// pack_ternary_bits (:131-153), dequantize_ternary (:182-207),
+// TernaryTensor::get_value (:275-291) in crates/ronn-providers/src/bitnet/.
+#include <cmath>
+#include <cstring>
+
+#include "common.hpp"
+#include "seqsum_core.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kSeqTile = 4096;  // elements per block map of the sequential sum (256 x 16)
+
+__device__ __forceinline__ uint32_t ternary_code(float v, float threshold) {
+    // quantization.rs:138-144.  NaN fails both comparisons and packs as 00 (-1).
+    return fabsf(v) <= threshold ? 1u : (v > 0.0f ? 2u : 0u);
+}
+
+// ---------------------------------------------------------------------------
+// pack_ternary_bits.  One thread per group of four consecutive elements makes one
+// byte; four neighbouring lanes merge their bytes into the little-endian u32 that
+// lane%4==0 stores.  A block covers 4096 elements in four strided passes so that
+// every load instruction of a wave reads 1 KiB of consecutive floats.
+// `survivors` (optional) receives the number of elements with |x| > threshold.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void pack_ternary_kernel(
+    const float *__restrict__ x, uint64_t n, float threshold, uint32_t *__restrict__ packed,
+    unsigned long long *__restrict__ survivors) {
+    const uint64_t n_quads = (n + 3) / 4;
+    const uint64_t n_words = (n + 15) / 16;
+    const uint64_t tile_quad0 = (uint64_t)blockIdx.x * (kBlock * 4);
+    float4 v[4];
+    bool full[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint64_t q = tile_quad0 + (uint64_t)j * kBlock + threadIdx.x;
+        full[j] = (q * 4 + 3) < n;
+        v[j] = full[j] ? reinterpret_cast<const float4 *>(x)[q] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    unsigned count = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint64_t q = tile_quad0 + (uint64_t)j * kBlock + threadIdx.x;
+        uint32_t byte = 0;
+        if (full[j]) {
+            float e[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                byte |= ternary_code(e[i], threshold) << (2 * i);
+                count += fabsf(e[i]) > threshold ? 1u : 0u;
+            }
+        } else if (q < n_quads) {  // the single partial group at the tail
+            for (int i = 0; i < 4; ++i) {
+                uint64_t idx = q * 4 + i;
+                if (idx < n) {
+                    float e = x[idx];
+                    byte |= ternary_code(e, threshold) << (2 * i);
+                    count += fabsf(e) > threshold ? 1u : 0u;
+                }
+            }
+        }
+        uint32_t word = byte << (8 * (threadIdx.x & 3));
+        word |= __shfl_xor(word, 1);
+        word |= __shfl_xor(word, 2);
+        if ((threadIdx.x & 3) == 0 && (q >> 2) < n_words) packed[q >> 2] = word;
+    }
+    if (survivors) {
+        // wave sum, then one atomic per wave (integer: order does not matter)
+        for (int off = 32; off > 0; off >>= 1) count += __shfl_down(count, off);
+        if ((threadIdx.x & 63) == 0 && count) atomicAdd(survivors, (unsigned long long)count);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Tree mode: deterministic f64 sum of |x| (optionally masked) and survivor count.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void abs_sum_tree_partial_kernel(
+    const float *__restrict__ x, uint64_t n, int use_mask, float thr, double *__restrict__ psum,
+    unsigned long long *__restrict__ pcnt) {
+    __shared__ double s_sum[kBlock];
+    __shared__ unsigned long long s_cnt[kBlock];
+    double acc = 0.0;
+    unsigned long long cnt = 0;
+    uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+        float a = fabsf(x[i]);
+        bool take = use_mask ? (a > thr) : true;
+        if (take) {
+            acc += (double)a;
+            ++cnt;
+        }
+    }
+    s_sum[threadIdx.x] = acc;
+    s_cnt[threadIdx.x] = cnt;
+    __syncthreads();
+    for (int off = kBlock / 2; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) {
+            s_sum[threadIdx.x] += s_sum[threadIdx.x + off];
+            s_cnt[threadIdx.x] += s_cnt[threadIdx.x + off];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        psum[blockIdx.x] = s_sum[0];
+        pcnt[blockIdx.x] = s_cnt[0];
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void abs_sum_tree_final_kernel(
+    const double *__restrict__ psum, const unsigned long long *__restrict__ pcnt, int nparts,
+    float *__restrict__ out_sum, unsigned long long *__restrict__ out_cnt) {
+    __shared__ double s_sum[kBlock];
+    __shared__ unsigned long long s_cnt[kBlock];
+    double acc = 0.0;
+    unsigned long long cnt = 0;
+    for (int i = threadIdx.x; i < nparts; i += kBlock) {
+        acc += psum[i];
+        cnt += pcnt[i];
+    }
+    s_sum[threadIdx.x] = acc;
+    s_cnt[threadIdx.x] = cnt;
+    __syncthreads();
+    for (int off = kBlock / 2; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) {
+            s_sum[threadIdx.x] += s_sum[threadIdx.x + off];
+            s_cnt[threadIdx.x] += s_cnt[threadIdx.x + off];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        *out_sum = (float)s_sum[0];
+        *out_cnt = s_cnt[0];
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Strict mode: the three kernels of the exact sequential sum (see seqsum_core.h).
+// ---------------------------------------------------------------------------
+struct SeqState {
+    uint32_t s_bits;       // current sum S as f32 bits (S >= 0)
+    uint32_t cross_block;  // window-relative block in which S leaves its binade, or ~0u
+    uint32_t k;            // integer state entering cross_block, or after the window
+    uint32_t next_rel;     // window-relative block at which the next window starts
+    uint32_t saw_nan;      // set by any_nan_kernel
+    uint32_t pad[3];
+};
+
+// One SeqMap per block of 4096 elements, valid for a state of biased exponent `es`.
+__global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
+    const float *__restrict__ x, uint64_t first, uint64_t n, uint32_t es, int use_mask,
+    float thr, SeqMap *__restrict__ maps) {
+    __shared__ SeqMap s_wave[kBlock / 64];
+    uint64_t base = first + (uint64_t)blockIdx.x * kSeqTile + (uint64_t)threadIdx.x * 16;
+    SeqMap m = seq_identity();
+    if (base + 16 <= n) {
+        float4 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = reinterpret_cast<const float4 *>(x + base)[j];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            float e[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float a = fabsf(e[i]);
+                bool take = use_mask ? (a > thr) : true;
+                if (take) m = seq_append(m, __float_as_uint(a), es);
+            }
+        }
+    } else {
+        for (int i = 0; i < 16; ++i) {
+            uint64_t idx = base + i;
+            if (idx < n) {
+                float a = fabsf(x[idx]);
+                bool take = use_mask ? (a > thr) : true;
+                if (take) m = seq_append(m, __float_as_uint(a), es);
+            }
+        }
+    }
+    // ordered tree over the wave: lane l absorbs lane l+off (its right neighbour)
+    for (int off = 1; off < 64; off <<= 1) {
+        SeqMap o;
+        o.d0 = __shfl_down(m.d0, off);
+        o.d1 = __shfl_down(m.d1, off);
+        m = seq_compose(m, o);
+    }
+    if ((threadIdx.x & 63) == 0) s_wave[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        SeqMap t = s_wave[0];
+        for (int w = 1; w < kBlock / 64; ++w) t = seq_compose(t, s_wave[w]);
+        maps[blockIdx.x] = t;
+    }
+}
+
+// Walks the block maps of a window from the true state and finds the first block
+// in which k reaches 2^24.  One workgroup of 1024 threads.
+__global__ __launch_bounds__(1024) void seq_scan_kernel(const SeqMap *__restrict__ maps,
+                                                        uint32_t nblocks,
+                                                        SeqState *__restrict__ state) {
+    __shared__ SeqMap s_a[1024];
+    __shared__ SeqMap s_b[1024];
+    __shared__ unsigned s_first;
+    const uint32_t t = threadIdx.x;
+    uint32_t es, k0;
+    seq_state_split(state->s_bits, &es, &k0);
+    const uint32_t chunk = (nblocks + 1023u) / 1024u;
+    const uint32_t lo = t * chunk;
+    const uint32_t hi = lo + chunk < nblocks ? lo + chunk : nblocks;
+    SeqMap mine = seq_identity();
+    for (uint32_t b = lo; b < hi; ++b) mine = seq_compose(mine, maps[b]);
+    if (t == 0) s_first = 0xffffffffu;
+    s_a[t] = mine;
+    __syncthreads();
+    // inclusive Hillis-Steele scan of the per-thread maps (order preserved)
+    SeqMap *src = s_a, *dst = s_b;
+    for (uint32_t off = 1; off < 1024u; off <<= 1) {
+        SeqMap v = src[t];
+        if (t >= off) v = seq_compose(src[t - off], v);
+        dst[t] = v;
+        __syncthreads();
+        SeqMap *tmp = src;
+        src = dst;
+        dst = tmp;
+    }
+    SeqMap before = t == 0 ? seq_identity() : src[t - 1];
+    uint32_t k = seq_apply(before, k0);
+    uint32_t cand = 0xffffffffu, cand_k = 0;
+    if (k < SEQ_K_LIMIT) {
+        for (uint32_t b = lo; b < hi; ++b) {
+            uint32_t k2 = seq_apply(maps[b], k);
+            if (k2 >= SEQ_K_LIMIT) {
+                cand = b;
+                cand_k = k;
+                break;
+            }
+            k = k2;
+        }
+    }
+    if (cand != 0xffffffffu) atomicMin(&s_first, cand);
+    __syncthreads();
+    const uint32_t first = s_first;
+    if (first != 0xffffffffu) {
+        if (cand == first) {
+            state->cross_block = first;
+            state->k = cand_k;
+        }
+    } else if (hi == nblocks && lo < hi) {
+        // this thread owns the last block of the window: k is the state after it
+        state->cross_block = 0xffffffffu;
+        state->k = k;
+    }
+}
+
+// Replays the crossing block with ordinary f32 additions (one wave; lane 0 adds).
+__global__ __launch_bounds__(64) void seq_replay_kernel(const float *__restrict__ x,
+                                                        uint64_t first, uint64_t n,
+                                                        uint32_t nblocks, int use_mask,
+                                                        float thr,
+                                                        SeqState *__restrict__ state) {
+    __shared__ float s_x[kSeqTile];
+    uint32_t es, k0;
+    seq_state_split(state->s_bits, &es, &k0);
+    const uint32_t cb = state->cross_block;
+    if (cb == 0xffffffffu) {
+        if (threadIdx.x == 0) {
+            state->s_bits = seq_state_join(es, state->k);
+            state->next_rel = nblocks;
+        }
+        return;
+    }
+    const uint64_t base = first + (uint64_t)cb * kSeqTile;
+    for (int i = threadIdx.x; i < kSeqTile; i += 64) {
+        uint64_t idx = base + i;
+        float a = 0.0f;
+        bool take = false;
+        if (idx < n) {
+            a = fabsf(x[idx]);
+            take = use_mask ? (a > thr) : true;
+        }
+        // a skipped element adds +0.0, which leaves any S >= 0 (and NaN/Inf) unchanged
+        s_x[i] = take ? a : 0.0f;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float s = __uint_as_float(seq_state_join(es, state->k));
+#pragma unroll 8
+        for (int i = 0; i < kSeqTile; ++i) s = s + s_x[i];
+        state->s_bits = __float_as_uint(s);
+        state->next_rel = cb + 1;
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void any_nan_kernel(const float *__restrict__ x,
+                                                         uint64_t first, uint64_t n,
+                                                         SeqState *__restrict__ state) {
+    uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    bool found = false;
+    for (uint64_t i = first + (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride)
+        found |= (x[i] != x[i]);
+    if (found) atomicOr(&state->saw_nan, 1u);
+}
+
+// ---------------------------------------------------------------------------
+// dequantize_ternary, get_value expansion, weight tiling
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ int ternary_value(uint32_t code) {
+    // quantization.rs:285-290: 00 -> -1, 01 -> 0, 10 -> +1, 11 -> 0
+    return code == 0u ? -1 : (code == 2u ? 1 : 0);
+}
+
+__global__ __launch_bounds__(kBlock) void dequantize_ternary_kernel(
+    const uint8_t *__restrict__ packed, uint64_t n, float scale, float *__restrict__ out) {
+    uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
+        uint32_t code = (packed[i >> 2] >> ((i & 3) * 2)) & 3u;
+        out[i] = code == 0u ? -scale : (code == 2u ? scale : 0.0f);
+    }
+}
+
+// One block per row: q[r, c] = get_value(r*cols + c), zero beyond cols; rowsum[r].
+__global__ __launch_bounds__(kBlock) void unpack_ternary_i8_kernel(
+    const uint8_t *__restrict__ packed, uint64_t cols, uint64_t pitch, int8_t *__restrict__ q,
+    int32_t *__restrict__ rowsum) {
+    __shared__ int s_sum[kBlock];
+    const uint64_t r = blockIdx.x;
+    int acc = 0;
+    for (uint64_t c = threadIdx.x; c < pitch; c += kBlock) {
+        int v = 0;
+        if (c < cols) {
+            uint64_t i = r * cols + c;
+            v = ternary_value((packed[i >> 2] >> ((i & 3) * 2)) & 3u);
+        }
+        q[r * pitch + c] = (int8_t)v;
+        acc += v;
+    }
+    s_sum[threadIdx.x] = acc;
+    __syncthreads();
+    for (int off = kBlock / 2; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) s_sum[threadIdx.x] += s_sum[threadIdx.x + off];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0 && rowsum) rowsum[r] = s_sum[0];
+}
+
+// "packed" [K,N] -> "tiled" [Kpad/16][Npad] words; see the header for the bit layout.
+__global__ __launch_bounds__(kBlock) void tile_weights_kernel(
+    const uint8_t *__restrict__ packed, uint64_t K, uint64_t N, uint64_t npad, uint64_t n_words,
+    uint32_t *__restrict__ tiled) {
+    uint64_t w = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (w >= n_words) return;
+    uint64_t kb = w / npad, n = w % npad;
+    uint32_t word = 0;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            uint64_t k = kb * 16 + 4 * s + b;
+            uint32_t code = 1u;  // padding is a zero weight
+            if (k < K && n < N) {
+                uint64_t i = k * N + n;
+                code = (packed[i >> 2] >> ((i & 3) * 2)) & 3u;
+                if (code == 3u) code = 1u;  // invalid pattern reads as zero
+            }
+            word |= code << (8 * b + 2 * s);
+        }
+    }
+    tiled[w] = word;
+}
+
+// Device scalars used by the reductions, at the start of the context workspace.
+struct ReduceScratch {
+    SeqState seq;
+    unsigned long long survivors;
+    float tree_sum;
+    uint32_t pad0;
+    unsigned long long tree_cnt;
+};
+constexpr size_t kScratchHeader = 256;
+static_assert(sizeof(ReduceScratch) <= kScratchHeader, "scratch header too small");
+constexpr int kTreeParts = 2048;
+
+inline bool is_finite_bits(uint32_t b) { return ((b >> 23) & 0xffu) != 0xffu; }
+
+// Exact sequential sum (optionally masked) of |x| over n elements.
+int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, float thr,
+                   float *h_sum) {
+    if (n == 0) {
+        *h_sum = -0.0f;  // Rust's empty f32 sum
+        return RBN_OK;
+    }
+    const uint64_t total_blocks = (n + kSeqTile - 1) / kSeqTile;
+    void *ws = nullptr;
+    RBN_CHECK(rbn_workspace(ctx, kScratchHeader + total_blocks * sizeof(SeqMap), &ws));
+    ReduceScratch *scr = (ReduceScratch *)ws;
+    SeqMap *maps = (SeqMap *)((char *)ws + kScratchHeader);
+    SeqState *h_state = (SeqState *)ctx->mailbox;
+    memset(h_state, 0, sizeof(SeqState));
+    RBN_HIP(hipMemcpyAsync(&scr->seq, h_state, sizeof(SeqState), hipMemcpyHostToDevice,
+                           ctx->stream));
+    RBN_HIP(hipStreamSynchronize(ctx->stream));
+    uint64_t pos = 0;  // in blocks
+    uint32_t s_bits = 0;
+    while (pos < total_blocks) {
+        if (!is_finite_bits(s_bits)) break;
+        uint32_t es, k;
+        seq_state_split(s_bits, &es, &k);
+        uint64_t win = pos + pos / 2;
+        if (win < 64) win = 64;
+        if (win > total_blocks - pos) win = total_blocks - pos;
+        const uint64_t first = pos * kSeqTile;
+        seq_block_maps_kernel<<<dim3((unsigned)win), dim3(kBlock), 0, ctx->stream>>>(
+            d_x, first, n, es, use_mask, thr, maps);
+        seq_scan_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(maps, (uint32_t)win, &scr->seq);
+        seq_replay_kernel<<<dim3(1), dim3(64), 0, ctx->stream>>>(d_x, first, n, (uint32_t)win,
+                                                                 use_mask, thr, &scr->seq);
+        RBN_HIP(hipGetLastError());
+        RBN_HIP(hipMemcpyAsync(h_state, &scr->seq, sizeof(SeqState), hipMemcpyDeviceToHost,
+                               ctx->stream));
+        RBN_HIP(hipStreamSynchronize(ctx->stream));
+        s_bits = h_state->s_bits;
+        if (h_state->next_rel == 0 || h_state->next_rel > win)
+            return rbn_fail(RBN_ERR_HIP, "sequential-sum scan made no progress (internal error)");
+        pos += h_state->next_rel;
+    }
+    float s;
+    memcpy(&s, &s_bits, 4);
+    if (!is_finite_bits(s_bits) && s == s && pos < total_blocks && !use_mask) {
+        // S is +Inf: it stays +Inf unless a NaN follows (masked sums never take a NaN).
+        any_nan_kernel<<<dim3(1024), dim3(kBlock), 0, ctx->stream>>>(d_x, pos * kSeqTile, n,
+                                                                     &scr->seq);
+        RBN_HIP(hipGetLastError());
+        RBN_HIP(hipMemcpyAsync(h_state, &scr->seq, sizeof(SeqState), hipMemcpyDeviceToHost,
+                               ctx->stream));
+        RBN_HIP(hipStreamSynchronize(ctx->stream));
+        if (h_state->saw_nan) s = NAN;
+    }
+    *h_sum = s;
+    return RBN_OK;
+}
+
+int tree_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, float thr,
+                 float *h_sum, uint64_t *h_count) {
+    if (n == 0) {
+        *h_sum = -0.0f;
+        if (h_count) *h_count = 0;
+        return RBN_OK;
+    }
+    void *ws = nullptr;
+    RBN_CHECK(rbn_workspace(ctx, kScratchHeader + kTreeParts * 16, &ws));
+    ReduceScratch *scr = (ReduceScratch *)ws;
+    double *psum = (double *)((char *)ws + kScratchHeader);
+    unsigned long long *pcnt = (unsigned long long *)(psum + kTreeParts);
+    uint64_t want = (n + kSeqTile - 1) / kSeqTile;
+    int parts = (int)(want < (uint64_t)kTreeParts ? want : (uint64_t)kTreeParts);
+    abs_sum_tree_partial_kernel<<<dim3(parts), dim3(kBlock), 0, ctx->stream>>>(d_x, n, use_mask,
+                                                                              thr, psum, pcnt);
+    abs_sum_tree_final_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(
+        psum, pcnt, parts, &scr->tree_sum, &scr->tree_cnt);
+    RBN_HIP(hipGetLastError());
+    char *mb = (char *)ctx->mailbox;
+    RBN_HIP(hipMemcpyAsync(mb, &scr->tree_sum, 4, hipMemcpyDeviceToHost, ctx->stream));
+    RBN_HIP(hipMemcpyAsync(mb + 8, &scr->tree_cnt, 8, hipMemcpyDeviceToHost, ctx->stream));
+    RBN_HIP(hipStreamSynchronize(ctx->stream));
+    memcpy(h_sum, mb, 4);
+    if (h_count) memcpy(h_count, mb + 8, 8);
+    return RBN_OK;
+}
+
+// pack + survivor count (count returned through the mailbox when h_survivors != NULL)
+int pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold, uint8_t *d_packed,
+                 uint64_t *h_survivors) {
+    if (n == 0) {
+        if (h_survivors) *h_survivors = 0;
+        return RBN_OK;
+    }
+    unsigned long long *d_cnt = nullptr;
+    if (h_survivors) {
+        void *ws = nullptr;
+        RBN_CHECK(rbn_workspace(ctx, kScratchHeader, &ws));
+        d_cnt = &((ReduceScratch *)ws)->survivors;
+        memset(ctx->mailbox, 0, 8);
+        RBN_HIP(hipMemcpyAsync(d_cnt, ctx->mailbox, 8, hipMemcpyHostToDevice, ctx->stream));
+    }
+    uint64_t tiles = (n + kSeqTile - 1) / kSeqTile;
+    if (tiles > 0x7fffffffull) return rbn_fail(RBN_ERR_UNSUPPORTED, "tensor too large");
+    pack_ternary_kernel<<<dim3((unsigned)tiles), dim3(kBlock), 0, ctx->stream>>>(
+        d_x, n, threshold, (uint32_t *)d_packed, d_cnt);
+    RBN_HIP(hipGetLastError());
+    if (h_survivors) {
+        RBN_HIP(hipMemcpyAsync(ctx->mailbox, d_cnt, 8, hipMemcpyDeviceToHost, ctx->stream));
+        RBN_HIP(hipStreamSynchronize(ctx->stream));
+        memcpy(h_survivors, ctx->mailbox, 8);
+    }
+    return RBN_OK;
+}
+
+int check_f32_ptr(const float *p, const char *name) {
+    RBN_REQUIRE(p != nullptr, "%s is NULL", name);
+    RBN_REQUIRE(((uintptr_t)p & 15u) == 0, "%s must be 16-byte aligned", name);
+    return RBN_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rbn_abs_sum_f32(rbn_ctx *ctx, const float *d_x, uint64_t n, int mode, int use_mask,
+                    float mask_threshold, float *h_sum, uint64_t *h_count) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(h_sum != nullptr, "h_sum is NULL");
+    RBN_REQUIRE(mode == RBN_SUM_STRICT_SEQ || mode == RBN_SUM_TREE, "unknown sum mode %d", mode);
+    if (n > 0) RBN_CHECK(check_f32_ptr(d_x, "d_x"));
+    if (mode == RBN_SUM_TREE)
+        return tree_abs_sum(ctx, d_x, n, use_mask, mask_threshold, h_sum, h_count);
+    RBN_CHECK(strict_abs_sum(ctx, d_x, n, use_mask, mask_threshold, h_sum));
+    if (h_count) {
+        if (!use_mask) {
+            *h_count = n;
+        } else {
+            float unused;
+            RBN_CHECK(tree_abs_sum(ctx, d_x, n, 1, mask_threshold, &unused, h_count));
+        }
+    }
+    return RBN_OK;
+}
+
+int rbn_pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold,
+                     uint8_t *d_packed) {
+    RBN_ENTER(ctx);
+    if (n == 0) return RBN_OK;
+    RBN_CHECK(check_f32_ptr(d_x, "d_x"));
+    RBN_REQUIRE(d_packed && ((uintptr_t)d_packed & 3u) == 0, "d_packed must be 4-byte aligned");
+    return pack_ternary(ctx, d_x, n, threshold, d_packed, nullptr);
+}
+
+int rbn_quantize_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, int mode, uint8_t *d_packed,
+                         float *h_scale, float *h_threshold, uint64_t *h_survivors) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(h_scale && h_threshold, "h_scale / h_threshold is NULL");
+    RBN_REQUIRE(mode == RBN_SUM_STRICT_SEQ || mode == RBN_SUM_TREE, "unknown sum mode %d", mode);
+    if (n > 0) {
+        RBN_CHECK(check_f32_ptr(d_x, "d_x"));
+        RBN_REQUIRE(d_packed && ((uintptr_t)d_packed & 3u) == 0,
+                    "d_packed must be 4-byte aligned");
+    }
+    // quantization.rs:79: (sum / n as f32) * 0.7
+    float sum = 0.0f;
+    if (mode == RBN_SUM_TREE)
+        RBN_CHECK(tree_abs_sum(ctx, d_x, n, 0, 0.0f, &sum, nullptr));
+    else
+        RBN_CHECK(strict_abs_sum(ctx, d_x, n, 0, 0.0f, &sum));
+    volatile float mean = sum / (float)n;
+    volatile float threshold = mean * 0.7f;
+    // quantization.rs:100 (pack) and the survivor count of :82-91
+    uint64_t survivors = 0;
+    RBN_CHECK(pack_ternary(ctx, d_x, n, threshold, d_packed, &survivors));
+    // quantization.rs:93-97
+    float scale = 1.0f;
+    if (survivors != 0) {
+        float nz_sum = 0.0f;
+        if (mode == RBN_SUM_TREE)
+            RBN_CHECK(tree_abs_sum(ctx, d_x, n, 1, threshold, &nz_sum, nullptr));
+        else
+            RBN_CHECK(strict_abs_sum(ctx, d_x, n, 1, threshold, &nz_sum));
+        volatile float sc = nz_sum / (float)survivors;
+        scale = sc;
+    }
+    *h_scale = scale;
+    *h_threshold = threshold;
+    if (h_survivors) *h_survivors = survivors;
+    return RBN_OK;
+}
+
+int rbn_dequantize_ternary(rbn_ctx *ctx, const uint8_t *d_packed, uint64_t n, float scale,
+                           float *d_out) {
+    RBN_ENTER(ctx);
+    if (n == 0) return RBN_OK;
+    RBN_REQUIRE(d_packed && d_out, "null pointer in rbn_dequantize_ternary");
+    uint64_t blocks = (n + kBlock - 1) / kBlock;
+    if (blocks > 65536) blocks = 65536;
+    dequantize_ternary_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream>>>(
+        d_packed, n, scale, d_out);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+int rbn_unpack_ternary_i8(rbn_ctx *ctx, const uint8_t *d_packed, uint64_t rows, uint64_t cols,
+                          uint64_t pitch, int8_t *d_q, int32_t *d_rowsum) {
+    RBN_ENTER(ctx);
+    if (rows == 0) return RBN_OK;
+    RBN_REQUIRE(d_packed && d_q, "null pointer in rbn_unpack_ternary_i8");
+    RBN_REQUIRE(pitch >= cols && pitch > 0, "pitch %llu smaller than cols %llu",
+                (unsigned long long)pitch, (unsigned long long)cols);
+    RBN_REQUIRE(rows <= 0x7fffffffull, "too many rows");
+    unpack_ternary_i8_kernel<<<dim3((unsigned)rows), dim3(kBlock), 0, ctx->stream>>>(
+        d_packed, cols, pitch, d_q, d_rowsum);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+int rbn_tile_weights(rbn_ctx *ctx, const uint8_t *d_packed, uint64_t K, uint64_t N,
+                     uint32_t *d_tiled) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(K > 0 && N > 0, "K and N must be positive");
+    RBN_REQUIRE(d_packed && d_tiled, "null pointer in rbn_tile_weights");
+    RBN_REQUIRE(((uintptr_t)d_tiled & 15u) == 0, "d_tiled must be 16-byte aligned");
+    uint64_t npad = rbn_npad(N);
+    uint64_t n_words = rbn_kpad(K) / 16 * npad;
+    uint64_t blocks = (n_words + kBlock - 1) / kBlock;
+    RBN_REQUIRE(blocks <= 0x7fffffffull, "weight matrix too large");
+    tile_weights_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream>>>(
+        d_packed, K, N, npad, n_words, d_tiled);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,182 @@
+// Host replica of the device's exact sequential-sum driver (ronn_amd/csrc/ternarize.hip:
+// seq_block_maps_kernel, seq_scan_kernel, seq_replay_kernel, strict_abs_sum), built on
+// the same arithmetic header.  It lets the CPU test-suite check the algorithm against
+// a literal `s = s + |x|` loop on any input, without a GPU.
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <vector>
+
+#include "../../ronn_amd/csrc/seqsum_core.h"
+
+namespace {
+constexpr int kTile = 4096;
+
+SeqMap thread_map(const float *x, uint64_t base, uint64_t n, uint32_t es, int use_mask, float thr) {
+    SeqMap m = seq_identity();
+    for (int i = 0; i < 16; ++i) {
+        uint64_t idx = base + i;
+        if (idx < n) {
+            float a = std::fabs(x[idx]);
+            bool take = use_mask ? (a > thr) : true;
+            if (take) {
+                uint32_t bits;
+                std::memcpy(&bits, &a, 4);
+                m = seq_append(m, bits, es);
+            }
+        }
+    }
+    return m;
+}
+
+SeqMap block_map(const float *x, uint64_t first, uint64_t n, uint32_t es, int use_mask, float thr) {
+    SeqMap lanes[256];
+    for (int t = 0; t < 256; ++t) lanes[t] = thread_map(x, first + (uint64_t)t * 16, n, es, use_mask, thr);
+    SeqMap waves[4];
+    for (int w = 0; w < 4; ++w) {
+        SeqMap v[64];
+        for (int l = 0; l < 64; ++l) v[l] = lanes[w * 64 + l];
+        for (int off = 1; off < 64; off <<= 1) {
+            SeqMap nv[64];
+            for (int l = 0; l < 64; ++l) {
+                SeqMap o = (l + off < 64) ? v[l + off] : v[l];  // out-of-range shuffles return own value
+                nv[l] = seq_compose(v[l], o);
+            }
+            for (int l = 0; l < 64; ++l) v[l] = nv[l];
+        }
+        waves[w] = v[0];
+    }
+    SeqMap t = waves[0];
+    for (int w = 1; w < 4; ++w) t = seq_compose(t, waves[w]);
+    return t;
+}
+
+struct ScanResult {
+    uint32_t cross_block;
+    uint32_t k;
+};
+
+ScanResult scan(const std::vector<SeqMap> &maps, uint32_t s_bits) {
+    const uint32_t nblocks = (uint32_t)maps.size();
+    uint32_t es, k0;
+    seq_state_split(s_bits, &es, &k0);
+    const uint32_t chunk = (nblocks + 1023u) / 1024u;
+    std::vector<SeqMap> a(1024), b(1024);
+    for (uint32_t t = 0; t < 1024; ++t) {
+        uint32_t lo = t * chunk, hi = lo + chunk < nblocks ? lo + chunk : nblocks;
+        SeqMap mine = seq_identity();
+        for (uint32_t i = lo; i < hi; ++i) mine = seq_compose(mine, maps[i]);
+        a[t] = mine;
+    }
+    std::vector<SeqMap> *src = &a, *dst = &b;
+    for (uint32_t off = 1; off < 1024u; off <<= 1) {
+        for (uint32_t t = 0; t < 1024; ++t) {
+            SeqMap v = (*src)[t];
+            if (t >= off) v = seq_compose((*src)[t - off], v);
+            (*dst)[t] = v;
+        }
+        std::swap(src, dst);
+    }
+    ScanResult r{0xffffffffu, 0};
+    uint32_t first = 0xffffffffu;
+    std::vector<uint32_t> cand(1024, 0xffffffffu), cand_k(1024, 0), last_k(1024, 0);
+    for (uint32_t t = 0; t < 1024; ++t) {
+        uint32_t lo = t * chunk, hi = lo + chunk < nblocks ? lo + chunk : nblocks;
+        SeqMap before = t == 0 ? seq_identity() : (*src)[t - 1];
+        uint32_t k = seq_apply(before, k0);
+        if (k < SEQ_K_LIMIT) {
+            for (uint32_t i = lo; i < hi; ++i) {
+                uint32_t k2 = seq_apply(maps[i], k);
+                if (k2 >= SEQ_K_LIMIT) {
+                    cand[t] = i;
+                    cand_k[t] = k;
+                    break;
+                }
+                k = k2;
+            }
+        }
+        last_k[t] = k;
+        if (cand[t] < first) first = cand[t];
+    }
+    for (uint32_t t = 0; t < 1024; ++t) {
+        uint32_t lo = t * chunk, hi = lo + chunk < nblocks ? lo + chunk : nblocks;
+        if (first != 0xffffffffu) {
+            if (cand[t] == first) r = ScanResult{first, cand_k[t]};
+        } else if (hi == nblocks && lo < hi) {
+            r = ScanResult{0xffffffffu, last_k[t]};
+        }
+    }
+    return r;
+}
+}  // namespace
+
+extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr,
+                             uint64_t *iterations, uint64_t *elements_read) {
+    uint64_t iters = 0, read = 0;
+    if (n == 0) {
+        if (iterations) *iterations = 0;
+        if (elements_read) *elements_read = 0;
+        return -0.0f;
+    }
+    const uint64_t total_blocks = (n + kTile - 1) / kTile;
+    uint64_t pos = 0;
+    uint32_t s_bits = 0;
+    while (pos < total_blocks) {
+        if (((s_bits >> 23) & 0xff) == 0xff) break;
+        uint32_t es, k;
+        seq_state_split(s_bits, &es, &k);
+        uint64_t win = pos + pos / 2;
+        if (win < 64) win = 64;
+        if (win > total_blocks - pos) win = total_blocks - pos;
+        const uint64_t first = pos * kTile;
+        std::vector<SeqMap> maps(win);
+        for (uint64_t b = 0; b < win; ++b) maps[b] = block_map(x, first + b * kTile, n, es, use_mask, thr);
+        read += win * kTile;
+        ScanResult sr = scan(maps, s_bits);
+        uint32_t next_rel;
+        if (sr.cross_block == 0xffffffffu) {
+            s_bits = seq_state_join(es, sr.k);
+            next_rel = (uint32_t)win;
+        } else {
+            uint32_t jb = seq_state_join(es, sr.k);
+            float s;
+            std::memcpy(&s, &jb, 4);
+            uint64_t base = first + (uint64_t)sr.cross_block * kTile;
+            for (int i = 0; i < kTile; ++i) {
+                uint64_t idx = base + i;
+                float a = 0.0f;
+                bool take = false;
+                if (idx < n) {
+                    a = std::fabs(x[idx]);
+                    take = use_mask ? (a > thr) : true;
+                }
+                volatile float t = s + (take ? a : 0.0f);
+                s = t;
+            }
+            std::memcpy(&s_bits, &s, 4);
+            next_rel = sr.cross_block + 1;
+        }
+        pos += next_rel;
+        ++iters;
+    }
+    float s;
+    std::memcpy(&s, &s_bits, 4);
+    if (((s_bits >> 23) & 0xff) == 0xff && s == s && pos < total_blocks && !use_mask) {
+        for (uint64_t i = pos * kTile; i < n; ++i)
+            if (x[i] != x[i]) s = NAN;
+    }
+    if (iterations) *iterations = iters;
+    if (elements_read) *elements_read = read;
+    return s;
+}
+
+// The literal fold the reference performs (quantization.rs:79 / :96).
+extern "C" float seqsum_literal(const float *x, uint64_t n, int use_mask, float thr) {
+    volatile float s = -0.0f;
+    for (uint64_t i = 0; i < n; ++i) {
+        float a = std::fabs(x[i]);
+        bool take = use_mask ? (a > thr) : true;
+        if (take) s = s + a;
+    }
+    return s;
+}

@@ -1,0 +1,341 @@
+"""HIP kernels against the CPU oracle, through the C ABI, on a real MI355X.
+
+Bar: packed bytes, thresholds, scales, int8 activations and int32 accumulators are
+bit-exact; f32 outputs are bit-exact too (stricter than the 1e-6 relative the
+target asks for), because |acc| < 2^24 and the epilogue keeps the reference's
+multiplication order.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from ronn_amd import _lib
+from ronn_amd.device import synth_normal
+from util import bits, decode_tiled, epilogue, exact_int_matmul, oracle_weights, same_bits
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+KATS = json.load(open(os.path.join(HERE, "golden", "ternary_kats.json")))
+STRICT, TREE = _lib.SUM_STRICT_SEQ, _lib.SUM_TREE
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def device_quantize(ctx, x, mode=STRICT):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    d_x = ctx.to_device(x)
+    d_p, scale, thr, cnt = ctx.quantize_ternary(d_x, x.size, mode)
+    packed = d_p.download(np.uint8, (x.size + 3) // 4)
+    return d_p, packed, scale, thr, cnt
+
+
+# ---- golden vectors -------------------------------------------------------------------
+
+@pytest.mark.parametrize("kat", KATS["quantize"], ids=lambda k: k["name"])
+def test_kat_quantize(ctx, kat):
+    x = np.array(kat["data"], dtype=np.float32)
+    _, packed, scale, thr, _ = device_quantize(ctx, x)
+    assert bytes(packed).hex() == kat["packed_hex"]
+    assert bits(thr) == kat["threshold_bits"] and bits(scale) == kat["scale_bits"]
+
+
+@pytest.mark.parametrize("kat", KATS["matmul"], ids=lambda k: k["name"])
+def test_kat_execute(ctx, kat):
+    a = np.array(kat["a"], dtype=np.float32).reshape(kat["m"], kat["k"])
+    b = np.array(kat["b"], dtype=np.float32).reshape(kat["k"], kat["n"])
+    out, acc = ctx.execute_ternary_matmul(a, b)
+    assert acc.ravel().tolist() == kat["acc"]
+    assert [bits(v) for v in out.ravel()] == kat["out_bits"]
+
+
+# ---- (1) ternarize + pack ----------------------------------------------------------------
+
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 15, 16, 17, 63, 64, 65, 4095, 4096, 4097, 100003])
+def test_pack_ragged_sizes(ctx, n):
+    x = synth_normal(100 + n, 1.0, (n,))
+    thr = np.float32(0.6)
+    d_p = ctx.pack_ternary(ctx.to_device(x), n, thr)
+    got = d_p.download(np.uint8, (n + 3) // 4)
+    assert (got == O.pack_ternary_bits(x, thr)).all()
+
+
+def test_pack_special_values(ctx):
+    x = np.array([-0.0, 0.0, np.nan, -np.nan, np.inf, -np.inf, 0.5, -0.5, 0.5000001, 1e-45] * 13,
+                 dtype=np.float32)
+    for thr in (np.float32(0.5), np.float32(0.0), np.float32(np.nan), np.float32(np.inf)):
+        got = ctx.pack_ternary(ctx.to_device(x), x.size, thr).download(np.uint8, (x.size + 3) // 4)
+        assert (got == O.pack_ternary_bits(x, thr)).all()
+
+
+DISTS = {
+    "weights_0.02": lambda n, s: synth_normal(s, 0.02, (n,)),
+    "acts_1.0": lambda n, s: synth_normal(s, 1.0, (n,)),
+    "ones": lambda n, s: np.ones(n, dtype=np.float32),
+    "zeros": lambda n, s: np.zeros(n, dtype=np.float32),
+    "denormal": lambda n, s: synth_normal(s, 1e-40, (n,)),
+    "huge": lambda n, s: synth_normal(s, 1e30, (n,)),
+    "wide": lambda n, s: (synth_normal(s, 1.0, (n,)) * np.exp(6 * synth_normal(s + 1, 1.0, (n,)))).astype(np.float32),
+}
+
+
+@pytest.mark.parametrize("dist", sorted(DISTS))
+@pytest.mark.parametrize("n", [1, 17, 4096, 4097, 70001, 1 << 20])
+def test_strict_abs_sum_matches_sequential_fold(ctx, dist, n):
+    x = DISTS[dist](n, 7)
+    want = np.cumsum(np.abs(x), dtype=np.float32)[-1]   # numpy's f32 cumsum is the same left fold
+    got, cnt = ctx.abs_sum(ctx.to_device(x), n, STRICT)
+    assert bits(got) == bits(want) and cnt == n
+    thr = np.float32(np.median(np.abs(x)))
+    surv = np.abs(x)[np.abs(x) > thr]
+    want_m = np.cumsum(surv, dtype=np.float32)[-1] if surv.size else np.float32(0)
+    got_m, cnt_m = ctx.abs_sum(ctx.to_device(x), n, STRICT, mask_threshold=thr)
+    assert cnt_m == surv.size
+    if surv.size:
+        assert bits(got_m) == bits(want_m)
+
+
+def test_strict_abs_sum_nonfinite(ctx):
+    x = synth_normal(9, 1.0, (100000,))
+    for edit, want in (({5000: np.inf}, np.inf), ({5000: np.inf, 90000: np.nan}, np.nan),
+                       ({70000: np.nan}, np.nan), ({}, None)):
+        y = x.copy()
+        for i, v in edit.items():
+            y[i] = v
+        got, _ = ctx.abs_sum(ctx.to_device(y), y.size, STRICT)
+        ref = np.cumsum(np.abs(y), dtype=np.float32)[-1]
+        assert bits(got) == bits(ref) or (np.isnan(got) and np.isnan(ref))
+    y = synth_normal(10, 3e37, (100000,))   # the fold overflows to +Inf
+    got, _ = ctx.abs_sum(ctx.to_device(y), y.size, STRICT)
+    assert np.isinf(got)
+
+
+def test_stall_at_two_pow_24(ctx):
+    n = (1 << 24) + 5000
+    got, _ = ctx.abs_sum(ctx.to_device(np.ones(n, dtype=np.float32)), n, STRICT)
+    assert got == np.float32(16777216.0)
+    tree, _ = ctx.abs_sum(ctx.to_device(np.ones(n, dtype=np.float32)), n, TREE)
+    assert tree == np.float32(n)
+
+
+@pytest.mark.parametrize("shape,sigma", [((64, 64), 0.02), ((2048, 2048), 0.02), ((1000, 777), 0.02),
+                                         ((4096, 4096), 0.02)])
+def test_quantize_ternary_bit_exact(ctx, shape, sigma):
+    w = synth_normal(0x5EED1001, sigma, shape)
+    say("quantize", shape)
+    t = O.quantize_ternary(w)
+    _, packed, scale, thr, cnt = device_quantize(ctx, w)
+    assert bits(thr) == bits(t.threshold)
+    assert cnt == t.survivors
+    assert bits(scale) == bits(t.scale)
+    assert (packed == t.packed_data).all()
+
+
+def test_quantize_tree_mode_is_close_but_flagged(ctx):
+    w = synth_normal(3, 0.02, (1 << 22,))
+    _, packed, scale, thr, cnt = device_quantize(ctx, w, TREE)
+    true_mean = np.abs(w).astype(np.float64).mean()
+    assert abs(float(thr) - 0.7 * true_mean) < 1e-7
+    surv = np.abs(w)[np.abs(w) > thr]
+    assert cnt == surv.size and abs(float(scale) - surv.astype(np.float64).mean()) < 1e-6
+    assert (packed == O.pack_ternary_bits(w, thr)).all()
+
+
+def test_quantize_edge_tensors(ctx):
+    for x in (np.zeros(10, dtype=np.float32), np.full(37, 3.0, dtype=np.float32),
+              np.array([np.nan, 1.0, -2.0, 0.25], dtype=np.float32)):
+        t = O.quantize_ternary(x)
+        _, packed, scale, thr, cnt = device_quantize(ctx, x)
+        assert (packed == t.packed_data).all() and cnt == t.survivors
+        assert bits(scale) == bits(t.scale)
+        assert bits(thr) == bits(t.threshold) or (np.isnan(thr) and np.isnan(t.threshold))
+    d_x = ctx.alloc(16)
+    d_p, scale, thr, cnt = ctx.quantize_ternary(d_x, 0)
+    assert np.isnan(thr) and scale == 1 and cnt == 0   # empty tensor
+
+
+def test_dequantize_and_unpack(ctx):
+    w = synth_normal(21, 0.02, (513,))
+    t = O.quantize_ternary(w)
+    d_p = ctx.to_device(np.concatenate([t.packed_data, np.zeros(32, np.uint8)]))
+    got = ctx.dequantize_ternary(d_p, w.size, t.scale).download(np.float32, w.size)
+    assert same_bits(got, O.dequantize_ternary(t))
+    # code 11 reads as zero (quantization.rs:195, :289)
+    raw = np.arange(256, dtype=np.uint8)
+    d_raw = ctx.to_device(np.concatenate([raw, np.zeros(32, np.uint8)]))
+    tt = O.TernaryTensor(raw, [1024], 2.0, 0.0, 1024)
+    assert same_bits(ctx.dequantize_ternary(d_raw, 1024, 2.0).download(np.float32, 1024),
+                     O.dequantize_ternary(tt))
+    d_q, d_r = ctx.unpack_ternary_i8(d_raw, 16, 64, 64)
+    vals = d_q.download(np.int8, 1024).reshape(16, 64)
+    assert (vals.ravel() == tt.values()).all()
+    assert (d_r.download(np.int32, 16) == vals.astype(np.int32).sum(1)).all()
+
+
+@pytest.mark.parametrize("K,N", [(3, 2), (16, 16), (64, 64), (100, 37), (130, 200), (256, 1376)])
+def test_tile_weights(ctx, K, N):
+    w = synth_normal(31, 0.02, (K, N))
+    t, vals = oracle_weights(w)
+    d_p = ctx.to_device(np.concatenate([t.packed_data, np.zeros(32, np.uint8)]))
+    d_t = ctx.tile_weights(d_p, K, N)
+    words = d_t.download(np.uint32, ctx.lib.rbn_tiled_bytes(K, N) // 4)
+    assert (decode_tiled(words, K, N) == vals).all()
+
+
+def test_tile_weights_sanitises_invalid_code(ctx):
+    raw = np.full(64 * 64 // 4, 0xFF, dtype=np.uint8)     # every field is 11
+    d_t = ctx.tile_weights(ctx.to_device(raw), 64, 64)
+    assert (decode_tiled(d_t.download(np.uint32, 64 * 64 // 16), 64, 64) == 0).all()
+
+
+# ---- (2) activation quantisation -----------------------------------------------------------
+
+@pytest.mark.parametrize("M,K", [(1, 2048), (1, 4096), (4, 11008), (16, 4096), (3, 100), (5, 1), (2, 67)])
+def test_act_quant_i8(ctx, M, K):
+    x = synth_normal(0x5EED0001, 1.0, (M, K))
+    if M >= 3:
+        x[1, :] = 0.0                  # zero token: guarded scale, all zeros
+        x[2, :] = x[2, :] * 1e-9
+    q, s, rs = O.act_quant_i8(x)
+    d_q, d_s, d_r = ctx.act_quant_i8(ctx.to_device(x), M, K)
+    pitch = ctx.act_pitch(K)
+    got = d_q.download(np.int8, M * pitch).reshape(M, pitch)
+    assert (got[:, :K] == q).all() and (got[:, K:] == 0).all()
+    assert same_bits(d_s.download(np.float32, M), s)
+    assert (d_r.download(np.int32, M) == rs).all()
+
+
+def test_act_quant_i8_ties_and_extremes(ctx):
+    x = np.array([[127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.49],
+                  [-127.0, 126.5, -126.5, 125.5, 0.49999997, -0.0, 1e-30, -1e-30]], dtype=np.float32)
+    q, s, rs = O.act_quant_i8(x)
+    d_q, d_s, d_r = ctx.act_quant_i8(ctx.to_device(x), 2, 8)
+    got = d_q.download(np.int8, 2 * 64).reshape(2, 64)[:, :8]
+    assert (got == q).all() and q[0].tolist() == [127, 0, 2, 2, 0, -2, -2, 3]
+    assert same_bits(d_s.download(np.float32, 2), s)
+
+
+@pytest.mark.parametrize("M,K", [(1, 2048), (4, 4096), (64, 64), (7, 99)])
+def test_act_quant_ternary_reference_mode(ctx, M, K):
+    x = synth_normal(0x5EED0002, 1.0, (M, K))
+    t = O.quantize_ternary(x)
+    d_q, d_s, d_r, scale, thr = ctx.act_quant_ternary(ctx.to_device(x), M, K)
+    pitch = ctx.act_pitch(K)
+    got = d_q.download(np.int8, M * pitch).reshape(M, pitch)
+    assert bits(scale) == bits(t.scale) and bits(thr) == bits(t.threshold)
+    assert (got[:, :K] == t.values().reshape(M, K)).all() and (got[:, K:] == 0).all()
+    assert same_bits(d_s.download(np.float32, M), np.full(M, t.scale, np.float32))
+    assert (d_r.download(np.int32, M) == got.astype(np.int32).sum(1)).all()
+
+
+# ---- (3)(4)(5) matmul ------------------------------------------------------------------------
+
+def run_matmul(ctx, fn, x, w, int8_acts=True):
+    """Device path from f32 inputs; returns (out, acc, q, act_scale, t_w)."""
+    M, K = x.shape
+    N = w.shape[1]
+    d_w = ctx.to_device(w)
+    d_p, w_scale, w_thr, _ = ctx.quantize_ternary(d_w, w.size)
+    d_t = ctx.tile_weights(d_p, K, N)
+    d_x = ctx.to_device(x)
+    if int8_acts:
+        acts = ctx.act_quant_i8(d_x, M, K)
+    else:
+        acts = ctx.act_quant_ternary(d_x, M, K)[:3]
+    d_out, d_acc = fn(acts, d_t, w_scale, M, K, N, want_acc=True)
+    pitch = ctx.act_pitch(K)
+    q = acts[0].download(np.int8, M * pitch).reshape(M, pitch)[:, :K]
+    s = acts[1].download(np.float32, M)
+    return (d_out.download(np.float32, M * N).reshape(M, N),
+            d_acc.download(np.int32, M * N).reshape(M, N), q, s, w_scale)
+
+
+def check_against_oracle(x, w, out, acc, q, s, w_scale, literal):
+    t, vals = oracle_weights(w)
+    assert bits(w_scale) == bits(t.scale)
+    if literal:   # the reference's own per-element loop
+        want_out, want_acc = O.matmul_i8_ternary(q, s, t)
+    else:         # same integers through BLAS (see util.exact_int_matmul)
+        want_acc = exact_int_matmul(q, vals)
+        want_out = epilogue(want_acc, s, t.scale)
+    assert (acc == want_acc).all()
+    assert same_bits(out, want_out)
+
+
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 8, 13, 16])
+@pytest.mark.parametrize("K,N", [(64, 64), (2048, 2048), (100, 37), (4096, 96), (130, 1376)])
+def test_gemv_small_literal(ctx, M, K, N):
+    say("gemv", M, K, N)
+    x = synth_normal(0x5EED0001 + M, 1.0, (M, K))
+    w = synth_normal(0x5EED1001 + K, 0.02, (K, N))
+    res = run_matmul(ctx, ctx.gemv, x, w)
+    check_against_oracle(x, w, *res, literal=(M * K * N <= 1 << 24))
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 11008), (11008, 4096)])
+def test_gemv_decode_sweep_shapes(ctx, M, K, N):
+    say("gemv sweep", M, K, N)
+    x = synth_normal(0x5EED0001 + M, 1.0, (M, K))
+    w = synth_normal(0x5EED1001 + N, 0.02, (K, N))
+    res = run_matmul(ctx, ctx.gemv, x, w)
+    check_against_oracle(x, w, *res, literal=(M == 1 and K * N <= 4096 * 4096))
+
+
+def test_gemv_reference_mode_config1(ctx):
+    # BASELINE config 1: x[1,2048] . W[2048,2048], both operands ternarised as the reference does
+    x = synth_normal(0x5EED0001, 1.0, (1, 2048))
+    w = synth_normal(0x5EED1001, 0.02, (2048, 2048))
+    want_out, want_acc = O.execute_ternary(x, w)
+    out, acc = ctx.execute_ternary_matmul(x, w)
+    assert (acc == want_acc).all() and same_bits(out, want_out)
+
+
+@pytest.mark.parametrize("M,K,N", [(17, 64, 64), (64, 64, 64), (128, 256, 128), (200, 130, 100),
+                                   (129, 4096, 257), (33, 100, 1376)])
+def test_gemm_mfma_small(ctx, M, K, N):
+    say("gemm", M, K, N)
+    x = synth_normal(0x5EED0003 + M, 1.0, (M, K))
+    w = synth_normal(0x5EED1003 + N, 0.02, (K, N))
+    res = run_matmul(ctx, ctx.gemm, x, w)
+    check_against_oracle(x, w, *res, literal=(M * K * N <= 1 << 23))
+
+
+def test_gemm_mfma_saturated_activations(ctx):
+    # every activation at +-127/-128 and dense +-1 weights: the largest |acc| the path can see
+    M, K, N = 64, 4096, 128
+    x = np.where(synth_normal(5, 1.0, (M, K)) > 0, 1.0, -1.0).astype(np.float32)
+    w = np.where(synth_normal(6, 1.0, (K, N)) > 0, 1.0, -1.0).astype(np.float32)
+    res = run_matmul(ctx, ctx.gemm, x, w)
+    check_against_oracle(x, w, *res, literal=False)
+    assert np.abs(res[1]).max() > 127 * 100
+
+
+def test_reference_execute_64_cubed(ctx):
+    # the only shape the reference's provider compiles kernels for (provider.rs:157-159)
+    a = synth_normal(41, 1.0, (64, 64))
+    b = synth_normal(42, 0.02, (64, 64))
+    want_out, want_acc = O.execute_ternary(a, b)
+    out, acc = ctx.execute_ternary_matmul(a, b)
+    assert (acc == want_acc).all() and same_bits(out, want_out)
+
+
+# ---- error behaviour ------------------------------------------------------------------------------
+
+def test_error_paths(ctx):
+    d = ctx.alloc(1024)
+    with pytest.raises(_lib.RbnError) as e:
+        ctx.gemv((d, d, d), d, 1.0, 17, 64, 64)
+    assert e.value.code == _lib.RBN_ERR_INVALID and "M <= 16" in e.value.message
+    with pytest.raises(_lib.RbnError):
+        ctx.gemv((d, d, d), d, 1.0, 0, 64, 64)
+    rc = ctx.lib.rbn_quantize_ternary(ctx.handle, d.ptr + 4, 16, 0, d.ptr, None, None, None)
+    assert rc == _lib.RBN_ERR_INVALID
+    rc = ctx.lib.rbn_gemv_t2_i8(ctx.handle, None, None, None, None, 1.0, 1, 64, 64, None, None)
+    assert rc == _lib.RBN_ERR_INVALID and b"null pointer" in ctx.lib.rbn_last_error()
+    assert ctx.lib.rbn_sync(None) == _lib.RBN_ERR_INVALID

@@ -120,6 +120,18 @@ size_t rbn_act_pitch(uint64_t K);
 int rbn_timer_start(rbn_ctx *ctx);
 int rbn_timer_stop(rbn_ctx *ctx, float *h_ms);
 
+/* ---- HIP graphs ----------------------------------------------------------- */
+/* Launch-bound sequences (a decode step is tens of kernels of a few microseconds)
+ * are captured once and replayed.  Between begin and end every asynchronous compute
+ * call on this context (pack, tile, act_quant_i8, gemv, gemm, matmul, d2d, fill) is
+ * recorded instead of run; calls that return scalars to the host or allocate are not
+ * allowed while capturing.  No reference counterpart. */
+typedef struct rbn_graph rbn_graph;
+int rbn_graph_begin_capture(rbn_ctx *ctx);
+int rbn_graph_end_capture(rbn_ctx *ctx, rbn_graph **out);
+int rbn_graph_launch(rbn_ctx *ctx, rbn_graph *graph);
+int rbn_graph_destroy(rbn_ctx *ctx, rbn_graph *graph);
+
 /* ---- (1) ternarize + pack: BitNetQuantizer::quantize_ternary,
  *      quantization.rs:67-109, and pack_ternary_bits, :131-153 -------------- */
 /* sum_i |x_i| in f32, as the reference's fold evaluates it (mode STRICT_SEQ) or

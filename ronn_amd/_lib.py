@@ -75,6 +75,10 @@ SIGNATURES = {
     "rbn_act_pitch": (C.c_size_t, [_u64]),
     "rbn_timer_start": (C.c_int, [_vp]),
     "rbn_timer_stop": (C.c_int, [_vp, _f32p]),
+    "rbn_graph_begin_capture": (C.c_int, [_vp]),
+    "rbn_graph_end_capture": (C.c_int, [_vp, C.POINTER(_vp)]),
+    "rbn_graph_launch": (C.c_int, [_vp, _vp]),
+    "rbn_graph_destroy": (C.c_int, [_vp, _vp]),
     "rbn_abs_sum_f32": (C.c_int, [_vp, _vp, _u64, C.c_int, C.c_int, C.c_float, _f32p, _u64p]),
     "rbn_pack_ternary": (C.c_int, [_vp, _vp, _u64, C.c_float, _vp]),
     "rbn_quantize_ternary": (C.c_int, [_vp, _vp, _u64, C.c_int, _vp, _f32p, _f32p, _u64p]),

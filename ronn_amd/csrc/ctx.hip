@@ -252,6 +252,59 @@ int rbn_timer_stop(rbn_ctx *ctx, float *h_ms) {
     return RBN_OK;
 }
 
+// ---- HIP graphs -----------------------------------------------------------------
+struct rbn_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+int rbn_graph_begin_capture(rbn_ctx *ctx) {
+    RBN_ENTER(ctx);
+    RBN_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+    return RBN_OK;
+}
+
+int rbn_graph_end_capture(rbn_ctx *ctx, rbn_graph **out) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(out != nullptr, "out is NULL");
+    *out = nullptr;
+    hipGraph_t g = nullptr;
+    RBN_HIP(hipStreamEndCapture(ctx->stream, &g));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+        (void)hipGraphDestroy(g);
+        return rbn_fail(RBN_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+    }
+    rbn_graph *r = new (std::nothrow) rbn_graph();
+    if (!r) {
+        (void)hipGraphExecDestroy(exec);
+        (void)hipGraphDestroy(g);
+        return rbn_fail(RBN_ERR_OOM, "host allocation failed");
+    }
+    r->graph = g;
+    r->exec = exec;
+    *out = r;
+    return RBN_OK;
+}
+
+int rbn_graph_launch(rbn_ctx *ctx, rbn_graph *graph) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(graph && graph->exec, "graph is NULL");
+    RBN_HIP(hipGraphLaunch(graph->exec, ctx->stream));
+    return RBN_OK;
+}
+
+int rbn_graph_destroy(rbn_ctx *ctx, rbn_graph *graph) {
+    RBN_ENTER(ctx);
+    if (!graph) return RBN_OK;
+    RBN_HIP(hipStreamSynchronize(ctx->stream));
+    if (graph->exec) (void)hipGraphExecDestroy(graph->exec);
+    if (graph->graph) (void)hipGraphDestroy(graph->graph);
+    delete graph;
+    return RBN_OK;
+}
+
 // ---- synthetic inputs ---------------------------------------------------------
 static inline uint64_t splitmix64_at(uint64_t seed, uint64_t index) {
     uint64_t z = seed + (index + 1) * 0x9E3779B97F4A7C15ull;

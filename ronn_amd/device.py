@@ -111,6 +111,21 @@ class Context:
         check(self.lib.rbn_timer_stop(self.handle, C.byref(ms)))
         return ms.value
 
+    # -- HIP graphs ------------------------------------------------------------------
+    def graph_begin(self):
+        check(self.lib.rbn_graph_begin_capture(self.handle))
+
+    def graph_end(self):
+        g = C.c_void_p()
+        check(self.lib.rbn_graph_end_capture(self.handle, C.byref(g)))
+        return g.value
+
+    def graph_launch(self, graph):
+        check(self.lib.rbn_graph_launch(self.handle, graph))
+
+    def graph_destroy(self, graph):
+        check(self.lib.rbn_graph_destroy(self.handle, graph))
+
     # -- (1) ternarize + pack ------------------------------------------------------
     def abs_sum(self, d_x: DeviceBuffer, n: int, mode=_lib.SUM_STRICT_SEQ, mask_threshold=None):
         s, cnt = C.c_float(), C.c_uint64()

@@ -26,13 +26,15 @@
  *             2*(i%4) of byte i/4; 00 = -1, 01 = 0, 10 = +1, 11 never produced and
  *             read as 0 (quantization.rs:285-290).  ceil(n/4) bytes; device buffers
  *             must have rbn_packed_capacity(n) bytes.
- *   "tiled"   Device-internal layout the matmul kernels stream: u32 word
- *             [kb][n], kb in [0,Kpad/16), n in [0,Npad), holds the 16 weights
- *             k = 16*kb + 4*s + b of column n as the 2-bit field at bit 8*b + 2*s
- *             (so (word >> 2*s) & 0x03030303 is four int8-ready codes of four
- *             consecutive k).  Code = value + 1 (same as "packed"); 11 and padding
- *             are stored as 01 (zero).  Kpad = K rounded up to 64, Npad = N rounded
- *             up to 64.  Built from "packed" by rbn_tile_weights().
+ *   "tiled"   Device-internal layout the matmul kernels stream.  Columns are grouped
+ *             in quads of four, k in blocks of sixteen.  The 16 bytes at uint4 index
+ *             q * KB + kb (KB = Kpad/16) are four u32 words, word c for column 4q+c;
+ *             a word holds the 16 weights k = 16*kb + 4*s + b of its column as the
+ *             2-bit field at bit 8*b + 2*s (so (word >> 2*s) & 0x03030303 is four
+ *             int8-ready codes of four consecutive k).  A quad's weights are thus
+ *             contiguous along k.  Code = value + 1 (same as "packed"); 11 and padding
+ *             are stored as 01 (zero).  Kpad = K rounded up to 64, Npad = N rounded up
+ *             to 64.  Built from "packed" by rbn_tile_weights().
  */
 #ifndef RONN_BITNET_HIP_H
 #define RONN_BITNET_HIP_H

@@ -36,7 +36,7 @@ __global__ __launch_bounds__(kThreads) void gemm_t2_i8_mfma_kernel(
     const int8_t *__restrict__ q,         // [M][Kpad]
     const float *__restrict__ act_scale,  // [M]
     const int32_t *__restrict__ rowsum,   // [M]
-    const uint32_t *__restrict__ wt,      // [Kpad/16][Npad]
+    const uint32_t *__restrict__ wt,      // tiled: word ((n/4) * Kpad/16 + kb) * 4 + n%4
     float w_scale, int M, int Kpad, int N, int Npad, int32_t *__restrict__ acc_out,
     float *__restrict__ out) {
     __shared__ __attribute__((aligned(16))) uint8_t s_a[2][BM * kRowStride];
@@ -72,6 +72,7 @@ __global__ __launch_bounds__(kThreads) void gemm_t2_i8_mfma_kernel(
     // B words of one k step of 64: [nt][ks]
     const int b_col = n0 + wn * 64 + (lane & 31);
     const int b_kgrp = lane >> 5;
+    const int kblocks = Kpad >> 4;
     auto load_b = [&](int k0, uint32_t (&w)[2][2]) {
 #pragma unroll
         for (int nt = 0; nt < 2; ++nt)
@@ -79,7 +80,8 @@ __global__ __launch_bounds__(kThreads) void gemm_t2_i8_mfma_kernel(
             for (int ks = 0; ks < 2; ++ks) {
                 int col = b_col + nt * 32;
                 int kb = (k0 >> 4) + ks * 2 + b_kgrp;
-                w[nt][ks] = col < Npad ? wt[(size_t)kb * Npad + col] : 0x55555555u;
+                w[nt][ks] = col < Npad ? wt[((size_t)(col >> 2) * kblocks + kb) * 4 + (col & 3)]
+                                       : 0x55555555u;
             }
     };
 

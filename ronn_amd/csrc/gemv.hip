@@ -5,145 +5,273 @@
 // crates/ronn-providers/src/bitnet/kernels.rs:134-178 (inner loop :161-165,
 // epilogue :168).
 //
-// The kernel is bound by HBM: it streams the tiled 2-bit weights exactly once with
-// 128-bit loads (four columns x sixteen k per lane and load), expands each word to
-// int8-ready bytes in registers ((w >> 2s) & 0x03030303) and accumulates with the
-// int8 dot instruction.  The weights are stored as code = value + 1, so
-//     sum_k q*w = sum_k q*code - sum_k q
-// and the per-token sum of q (rowsum) is subtracted once in the epilogue; this is
-// integer-exact.  One workgroup owns 32 columns for the whole of K: its 256 lanes
-// are 8 (columns/4) x 32 (k slices); partial sums meet through DPP/LDS, never
-// through global memory, and the epilogue is fused.
+// The kernel is bound by HBM.  Design, each point measured on an MI355X:
+//  * One wavefront owns one quad of four adjacent columns.  In the tiled layout a
+//    quad's weights are contiguous along k (16 bytes per 16 k), so every load
+//    instruction of a wave reads 1 KiB of consecutive memory and a workgroup reads
+//    a few consecutive KiB: the access pattern of a plain streaming read.
+//  * Lanes split k.  The partial sums of a wave meet through six DPP additions
+//    (quad_perm, row_ror, row_bcast); nothing crosses waves unless the matrix has too
+//    few columns to fill the chip, in which case KS waves share a quad's k range and
+//    meet through LDS.  Global memory is never used for partial sums.
+//  * Activations are issued to the memory pipe BEFORE the weights (the vector-memory
+//    counter retires in order) and staged in LDS once per workgroup, so the weight
+//    stream is the only traffic of any size.
+//  * Weights are stored as code = value + 1 in {0,1,2}.  Two VALU operations split a
+//    word into two registers of eight 4-bit codes ((w & 0x33333333),
+//    ((w >> 2) & 0x33333333)); the activations are staged as 4-bit planes
+//    (a = 16 * hi + lo, hi signed, lo unsigned) so that v_dot8_i32_i4 and
+//    v_dot8_u32_u4 consume them directly: 3 + 4 VALU operations per 16 weights
+//    instead of 7 + 4 with byte-wise v_dot4.  sum q*w = sum q*code - sum q; the
+//    per-token sum of q is subtracted once in the epilogue.  All of it is
+//    integer-exact.
 #include "common.hpp"
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kTN = 8;                   // lanes along n; each covers 4 columns
-constexpr int kTK = kThreads / kTN;      // 32 k-slices
-constexpr int kColsPerBlock = kTN * 4;   // 32
-// kIters weight loads are in flight per lane and chunk; a chunk spans kTK * kIters
-// k-blocks (8 -> 4096 k).  Sixteen tokens use 4 so that the activation chunk stays
-// within the 64 KiB of static LDS.
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int kLdsBudget = 48 * 1024;  // bytes of staged activations per workgroup
 
-__device__ __forceinline__ int dot4(uint32_t a, uint32_t b, int c) {
-    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ int dpp_add(int v) {
+    return v + __builtin_amdgcn_update_dpp(0, v, CTRL, ROWMASK, 0xf, false);
 }
 
-template <int MT, int kIters>
+// Sum over the 64 lanes of a wave; the total is valid in lane 63.
+__device__ __forceinline__ int wave_total_lane63(int v) {
+    v = dpp_add<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x124, 0xf>(v);  // row_ror:4
+    v = dpp_add<0x128, 0xf>(v);  // row_ror:8   -> every lane holds its row's total
+    v = dpp_add<0x142, 0xA>(v);  // row_bcast15 -> rows 1 and 3 add rows 0 and 2
+    v = dpp_add<0x143, 0xC>(v);  // row_bcast31 -> rows 2 and 3 add row 1
+    return v;
+}
+
+// int8 x16 (k = 0..15 of one 16-k block, natural order) -> the four 4-bit planes that
+// pair with the even/odd 2-bit fields of a tiled weight word:
+//   .x high nibbles, k order (0,8,1,9,2,10,3,11)   .y low nibbles, same order
+//   .z high nibbles, k order (4,12,5,13,6,14,7,15) .w low nibbles, same order
+__device__ __forceinline__ uint4 to_nibble_planes(uint4 a) {
+    uint4 p;
+    p.x = ((a.x >> 4) & 0x0F0F0F0Fu) | (a.z & 0xF0F0F0F0u);
+    p.y = (a.x & 0x0F0F0F0Fu) | ((a.z & 0x0F0F0F0Fu) << 4);
+    p.z = ((a.y >> 4) & 0x0F0F0F0Fu) | (a.w & 0xF0F0F0F0u);
+    p.w = (a.y & 0x0F0F0F0Fu) | ((a.w & 0x0F0F0F0Fu) << 4);
+    return p;
+}
+
+// MT tokens, KS waves per column quad, L weight loads in flight per lane and round.
+template <int MT, int KS, int L>
 __global__ __launch_bounds__(kThreads) void gemv_t2_i8_kernel(
-    const uint4 *__restrict__ q4,         // [M][KB] 16 int8 each
+    const uint4 *__restrict__ q4,         // [M][KB]: 16 int8 each
     const float *__restrict__ act_scale,  // [M]
     const int32_t *__restrict__ rowsum,   // [M]
-    const uint4 *__restrict__ w4,         // [KB][Npad/4]
-    float w_scale, int M, int KB, int N, int npad4, int32_t *__restrict__ acc_out,
-    float *__restrict__ out) {
-    constexpr int kChunkKb = kTK * kIters;
-    __shared__ uint4 s_a[MT * kChunkKb];             // activation chunk, MT x 4 KiB
-    __shared__ int s_red[kThreads / 64][MT][kColsPerBlock];
+    const uint4 *__restrict__ w4,         // [nquads][KB]
+    float w_scale, int M, int KB, int KC /* k-blocks staged per pass */, int N, int nquads,
+    int32_t *__restrict__ acc_out, float *__restrict__ out) {
+    constexpr int QPB = kWaves / KS;  // quads per workgroup
+    extern __shared__ uint4 s_a[];  // MT * KC staged activation blocks (4-bit planes)
+    __shared__ int s_part[KS > 1 ? kWaves * MT * 4 : 1];
 
     const int tid = threadIdx.x;
-    const int tn = tid & (kTN - 1);
-    const int tk = tid >> 3;
-    const int col4 = blockIdx.x * kTN + tn;  // < npad4 by construction of the grid
+    const int lane = tid & 63, wave = tid >> 6;
+    const int quad_local = wave / KS, slice = wave % KS;
+    int quad = blockIdx.x * QPB + quad_local;
+    const bool active = quad < nquads;
+    quad = active ? quad : nquads - 1;
+    const uint4 *wq = w4 + (size_t)quad * KB;
 
-    int acc[MT][4];
-#pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int c = 0; c < 4; ++c) acc[m][c] = 0;
-
-    for (int kc0 = 0; kc0 < KB; kc0 += kChunkKb) {
-        // 1. put this chunk's weight loads in flight
-        uint4 w[kIters];
-#pragma unroll
-        for (int it = 0; it < kIters; ++it) {
-            int kb = kc0 + it * kTK + tk;
-            w[it] = kb < KB ? w4[(size_t)kb * npad4 + col4]
-                            : make_uint4(0x55555555u, 0x55555555u, 0x55555555u, 0x55555555u);
-        }
-        // 2. stage the activations of the chunk in LDS
-        if (kc0 != 0) __syncthreads();
-        if (tid < kChunkKb) {
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                int kb = kc0 + tid;
-                uint4 a = make_uint4(0u, 0u, 0u, 0u);
-                if (m < M && kb < KB) a = q4[(size_t)m * KB + kb];
-                s_a[m * kChunkKb + tid] = a;
-            }
-        }
-        __syncthreads();
-        // 3. decode and accumulate
-#pragma unroll
-        for (int it = 0; it < kIters; ++it) {
-            const uint32_t ww[4] = {w[it].x, w[it].y, w[it].z, w[it].w};
-            uint32_t b[4][4];
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                b[c][0] = ww[c] & 0x03030303u;
-                b[c][1] = (ww[c] >> 2) & 0x03030303u;
-                b[c][2] = (ww[c] >> 4) & 0x03030303u;
-                b[c][3] = (ww[c] >> 6) & 0x03030303u;
-            }
-#pragma unroll
-            for (int m = 0; m < MT; ++m) {
-                const uint4 a = s_a[m * kChunkKb + it * kTK + tk];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    int v = acc[m][c];
-                    v = dot4(a.x, b[c][0], v);
-                    v = dot4(a.y, b[c][1], v);
-                    v = dot4(a.z, b[c][2], v);
-                    v = dot4(a.w, b[c][3], v);
-                    acc[m][c] = v;
-                }
-            }
-        }
-    }
-
-    // 4. reduce over the 32 k-slices: 8 inside the wave (lane bits 3..5), then 4 waves.
+    int hi[MT][4], lo[MT][4];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            int v = acc[m][c];
-            v += __shfl_xor(v, 8);
-            v += __shfl_xor(v, 16);
-            v += __shfl_xor(v, 32);
-            acc[m][c] = v;
+            hi[m][c] = 0;
+            lo[m][c] = 0;
         }
-    const int lane = tid & 63, wave = tid >> 6;
-    if (lane < kTN) {
+
+    for (int kc = 0; kc < KB; kc += KC) {
+        const int kc_len = min(KC, KB - kc);
+        // this wave's k range inside the pass
+        const int sl_len = (kc_len + KS - 1) / KS;
+        const int sl_lo = kc + slice * sl_len;
+        const int sl_hi = min(sl_lo + sl_len, kc + kc_len);
+
+        // (1) activations first, (2) the first round of weights, then the LDS hand-over.
+        // Every load below is unconditional (indices are clamped, never branched on) so
+        // that the compiler keeps them back to back and waits with vmcnt(L), not vmcnt(0).
+        const int n_stage = MT * kc_len;  // uint4 entries: [m][kb - kc]
+        constexpr int kPre = MT * KS * L / 4 < 1 ? 1 : (MT * KS * L / 4 > 4 ? 4 : MT * KS * L / 4);
+        uint4 stage[kPre];
 #pragma unroll
-        for (int m = 0; m < MT; ++m)
+        for (int j = 0; j < kPre; ++j) {
+            const int e = min(tid + j * kThreads, n_stage - 1);
+            const int m = MT == 1 ? 0 : min(e / kc_len, M - 1);  // spare token rows repeat the last
+            const int kb = kc + (MT == 1 ? e : e % kc_len);
+            stage[j] = q4[(size_t)m * KB + kb];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        uint4 w[L];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) s_red[wave][m][lane * 4 + c] = acc[m][c];
+        for (int it = 0; it < L; ++it) {
+            const int kb = sl_lo + it * 64 + lane;
+            // a lane past its slice re-reads its first block (a cache hit) and adds 0
+            w[it] = wq[kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (kc != 0) __syncthreads();  // everyone is done reading the previous pass
+#pragma unroll
+        for (int j = 0; j < kPre; ++j) {
+            const int e = tid + j * kThreads;
+            if (e < n_stage) s_a[e] = to_nibble_planes(stage[j]);
+        }
+        for (int e = tid + kPre * kThreads; e < n_stage; e += kThreads) {
+            const int m = min(e / kc_len, M - 1), kb = kc + e % kc_len;
+            s_a[e] = to_nibble_planes(q4[(size_t)m * KB + kb]);
+        }
+        __syncthreads();
+
+        // One round: expand L loaded blocks and accumulate.  Beyond the slice the codes are
+        // forced to 0, so the lane adds q * 0.
+        auto consume = [&](const uint4(&wr)[L], int r0) {
+#pragma unroll
+            for (int it = 0; it < L; ++it) {
+                const int kb = r0 + it * 64 + lane;
+                const uint32_t keep = kb < sl_hi ? 0x33333333u : 0u;
+                const int a_idx = min(kb, sl_hi - 1) - kc;
+                const uint32_t ww[4] = {wr[it].x, wr[it].y, wr[it].z, wr[it].w};
+                uint32_t ev[4], od[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    ev[c] = ww[c] & keep;
+                    od[c] = (ww[c] >> 2) & keep;
+                }
+#pragma unroll
+                for (int m = 0; m < MT; ++m) {
+                    const uint4 a = s_a[m * kc_len + a_idx];
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        hi[m][c] = __builtin_amdgcn_sdot8((int)a.x, (int)ev[c], hi[m][c], false);
+                        lo[m][c] = (int)__builtin_amdgcn_udot8(a.y, ev[c], (uint32_t)lo[m][c], false);
+                        hi[m][c] = __builtin_amdgcn_sdot8((int)a.z, (int)od[c], hi[m][c], false);
+                        lo[m][c] = (int)__builtin_amdgcn_udot8(a.w, od[c], (uint32_t)lo[m][c], false);
+                    }
+                }
+            }
+        };
+        // Rounds with a successor prefetch it before consuming; the last round has nothing
+        // else in flight, so its blocks are consumed as they arrive (vmcnt L-1, L-2, ...).
+        int r0 = sl_lo;
+        while (r0 + 64 * L < sl_hi) {
+            uint4 wn[L];
+#pragma unroll
+            for (int it = 0; it < L; ++it) {
+                const int kb = r0 + 64 * L + it * 64 + lane;
+                wn[it] = wq[kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)];
+            }
+            consume(w, r0);
+#pragma unroll
+            for (int it = 0; it < L; ++it) w[it] = wn[it];
+            r0 += 64 * L;
+        }
+        if (r0 < sl_hi) consume(w, r0);
     }
-    __syncthreads();
-    // 5. fused epilogue: one thread per (m, column)
-    for (int idx = tid; idx < MT * kColsPerBlock; idx += kThreads) {
-        int m = idx / kColsPerBlock, c = idx % kColsPerBlock;
-        int n = blockIdx.x * kColsPerBlock + c;
-        if (m < M && n < N) {
-            int total = s_red[0][m][c] + s_red[1][m][c] + s_red[2][m][c] + s_red[3][m][c];
-            total -= rowsum[m];
-            if (acc_out) acc_out[(size_t)m * N + n] = total;
-            float r = (float)total * act_scale[m];  // kernels.rs:168, left to right
-            r = r * w_scale;
-            out[(size_t)m * N + n] = r;
+
+    // wave totals (lane 63), then across the KS waves of a quad if any
+    int tot[MT][4];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int c = 0; c < 4; ++c) tot[m][c] = wave_total_lane63(hi[m][c] * 16 + lo[m][c]);
+
+    if (KS == 1) {
+        if (lane == 63 && active) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) {
+                if (m >= M) break;
+                const int rs = rowsum[m];
+                const float as = act_scale[m];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int n = quad * 4 + c;
+                    if (n < N) {
+                        const int total = tot[m][c] - rs;
+                        if (acc_out) acc_out[(size_t)m * N + n] = total;
+                        float r = (float)total * as;  // kernels.rs:168, left to right
+                        r = r * w_scale;
+                        out[(size_t)m * N + n] = r;
+                    }
+                }
+            }
+        }
+    } else {
+        if (lane == 63) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) s_part[(wave * MT + m) * 4 + c] = tot[m][c];
+        }
+        __syncthreads();
+        for (int idx = tid; idx < QPB * MT * 4; idx += kThreads) {
+            const int ql = idx / (MT * 4), m = (idx / 4) % MT, c = idx % 4;
+            const int qd = blockIdx.x * QPB + ql;
+            const int n = qd * 4 + c;
+            if (qd < nquads && m < M && n < N) {
+                int total = 0;
+#pragma unroll
+                for (int s = 0; s < KS; ++s) total += s_part[((ql * KS + s) * MT + m) * 4 + c];
+                total -= rowsum[m];
+                if (acc_out) acc_out[(size_t)m * N + n] = total;
+                float r = (float)total * act_scale[m];  // kernels.rs:168, left to right
+                r = r * w_scale;
+                out[(size_t)m * N + n] = r;
+            }
         }
     }
 }
 
+struct Args {
+    const uint4 *q4;
+    const float *act_scale;
+    const int32_t *rowsum;
+    const uint4 *w4;
+    float w_scale;
+    int M, KB, KC, N, nquads;
+    int32_t *acc;
+    float *out;
+};
+
+template <int MT, int KS, int L>
+void launch(hipStream_t stream, const Args &a) {
+    constexpr int QPB = kWaves / KS;
+    dim3 grid((unsigned)((a.nquads + QPB - 1) / QPB));
+    const size_t lds = (size_t)MT * a.KC * 16;
+    gemv_t2_i8_kernel<MT, KS, L><<<grid, dim3(kThreads), lds, stream>>>(
+        a.q4, a.act_scale, a.rowsum, a.w4, a.w_scale, a.M, a.KB, a.KC, a.N, a.nquads, a.acc, a.out);
+}
+
+template <int MT, int KS>
+void launch_l(hipStream_t stream, const Args &a, int loads) {
+    if (loads <= 1)
+        launch<MT, KS, 1>(stream, a);
+    else if (loads <= 2 || MT >= 8)
+        launch<MT, KS, 2>(stream, a);
+    else
+        launch<MT, KS, 4>(stream, a);
+}
+
 template <int MT>
-void launch(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale, const int32_t *d_rowsum,
-            const uint32_t *d_tiled, float w_scale, int M, int KB, int N, int npad4,
-            int32_t *d_acc, float *d_out) {
-    dim3 grid((unsigned)(npad4 / kTN));
-    gemv_t2_i8_kernel<MT, (MT >= 16 ? 4 : 8)><<<grid, dim3(kThreads), 0, ctx->stream>>>(
-        (const uint4 *)d_q, d_act_scale, d_rowsum, (const uint4 *)d_tiled, w_scale, M, KB, N,
-        npad4, d_acc, d_out);
+void launch_ks(hipStream_t stream, const Args &a, int ks) {
+    // weight loads per lane needed to cover one wave's share of a pass
+    const int sl_len = ((a.KC + ks - 1) / ks + 63) / 64;
+    if (ks == 4)
+        launch_l<MT, 4>(stream, a, sl_len);
+    else if (ks == 2)
+        launch_l<MT, 2>(stream, a, sl_len);
+    else
+        launch_l<MT, 1>(stream, a, sl_len);
 }
 
 }  // namespace
@@ -159,20 +287,33 @@ extern "C" int rbn_gemv_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_ac
     RBN_REQUIRE((((uintptr_t)d_q | (uintptr_t)d_tiled) & 15u) == 0,
                 "d_q and d_tiled must be 16-byte aligned");
     RBN_REQUIRE(K <= (1ull << 30) && N <= (1ull << 30), "dimension too large");
-    const int KB = (int)(rbn_kpad(K) / 16);
-    const int npad4 = (int)(rbn_npad(N) / 4);
-    const int m = (int)M, n = (int)N;
-    if (m == 1)
-        launch<1>(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, m, KB, n, npad4, d_acc, d_out);
-    else if (m == 2)
-        launch<2>(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, m, KB, n, npad4, d_acc, d_out);
-    else if (m <= 4)
-        launch<4>(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, m, KB, n, npad4, d_acc, d_out);
-    else if (m <= 8)
-        launch<8>(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, m, KB, n, npad4, d_acc, d_out);
-    else
-        launch<16>(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, m, KB, n, npad4, d_acc,
-                   d_out);
+    Args a;
+    a.q4 = (const uint4 *)d_q;
+    a.act_scale = d_act_scale;
+    a.rowsum = d_rowsum;
+    a.w4 = (const uint4 *)d_tiled;
+    a.w_scale = w_scale;
+    a.M = (int)M;
+    a.KB = (int)(rbn_kpad(K) / 16);
+    a.N = (int)N;
+    a.nquads = (int)(rbn_npad(N) / 4);
+    a.acc = d_acc;
+    a.out = d_out;
+    const int mt = M == 1 ? 1 : M == 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
+    // k-blocks whose staged activations fit the LDS budget in one pass
+    const int kc_cap = kLdsBudget / 16 / mt;
+    a.KC = a.KB < kc_cap ? a.KB : kc_cap;
+    // Waves per quad: enough wavefronts to cover the chip (256 CUs x 4 SIMDs, a few waves
+    // each) without shrinking a wave's share of k below one round.
+    int ks = 1;
+    while (ks < 4 && (long long)a.nquads * ks < 2048 && a.KB / (ks * 2) >= 128) ks *= 2;
+    switch (mt) {
+        case 1: launch_ks<1>(ctx->stream, a, ks); break;
+        case 2: launch_ks<2>(ctx->stream, a, ks); break;
+        case 4: launch_ks<4>(ctx->stream, a, ks); break;
+        case 8: launch_ks<8>(ctx->stream, a, ks); break;
+        default: launch_ks<16>(ctx->stream, a, ks); break;
+    }
     RBN_HIP(hipGetLastError());
     return RBN_OK;
 }

@@ -346,13 +346,15 @@ __global__ __launch_bounds__(kBlock) void unpack_ternary_i8_kernel(
     if (threadIdx.x == 0 && rowsum) rowsum[r] = s_sum[0];
 }
 
-// "packed" [K,N] -> "tiled" [Kpad/16][Npad] words; see the header for the bit layout.
+// "packed" [K,N] -> "tiled": u32 word ((q * KB + kb) * 4 + c) holds column 4q+c, k-block kb;
+// see the header for the bit layout inside a word.
 __global__ __launch_bounds__(kBlock) void tile_weights_kernel(
-    const uint8_t *__restrict__ packed, uint64_t K, uint64_t N, uint64_t npad, uint64_t n_words,
+    const uint8_t *__restrict__ packed, uint64_t K, uint64_t N, uint64_t kblocks, uint64_t n_words,
     uint32_t *__restrict__ tiled) {
     uint64_t w = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
     if (w >= n_words) return;
-    uint64_t kb = w / npad, n = w % npad;
+    const uint64_t q = w / (kblocks * 4), rem = w % (kblocks * 4);
+    const uint64_t kb = rem >> 2, n = q * 4 + (rem & 3);
     uint32_t word = 0;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
@@ -608,12 +610,12 @@ int rbn_tile_weights(rbn_ctx *ctx, const uint8_t *d_packed, uint64_t K, uint64_t
     RBN_REQUIRE(K > 0 && N > 0, "K and N must be positive");
     RBN_REQUIRE(d_packed && d_tiled, "null pointer in rbn_tile_weights");
     RBN_REQUIRE(((uintptr_t)d_tiled & 15u) == 0, "d_tiled must be 16-byte aligned");
-    uint64_t npad = rbn_npad(N);
-    uint64_t n_words = rbn_kpad(K) / 16 * npad;
+    uint64_t kblocks = rbn_kpad(K) / 16;
+    uint64_t n_words = kblocks * rbn_npad(N);
     uint64_t blocks = (n_words + kBlock - 1) / kBlock;
     RBN_REQUIRE(blocks <= 0x7fffffffull, "weight matrix too large");
     tile_weights_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream>>>(
-        d_packed, K, N, npad, n_words, d_tiled);
+        d_packed, K, N, kblocks, n_words, d_tiled);
     RBN_HIP(hipGetLastError());
     return RBN_OK;
 }

@@ -39,10 +39,16 @@ def epilogue(acc, act_scale, w_scale):
 
 
 def decode_tiled(tiled_words, K, N):
-    """Inverse of the device's weight tiling: u32 [Kpad/16, Npad] -> int8 values [K, N]."""
+    """Inverse of the device's weight tiling: u32 words -> int8 values [K, N].
+
+    Word ((q * KB + kb) * 4 + c) belongs to column 4q+c and k-block kb; inside a word the
+    weight k = 16*kb + 4*s + b sits at bit 8*b + 2*s as code = value + 1.
+    """
     kpad = (K + 63) // 64 * 64
     npad = (N + 63) // 64 * 64
-    t = np.asarray(tiled_words, dtype=np.uint32).reshape(kpad // 16, npad)
+    kb_n = kpad // 16
+    t = np.asarray(tiled_words, dtype=np.uint32).reshape(npad // 4, kb_n, 4)
+    t = t.transpose(1, 0, 2).reshape(kb_n, npad)          # [kb][column]
     out = np.zeros((kpad, npad), dtype=np.int8)
     for s in range(4):
         for b in range(4):

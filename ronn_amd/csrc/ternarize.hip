@@ -29,49 +29,60 @@ __device__ __forceinline__ uint32_t ternary_code(float v, float threshold) {
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(kBlock) void pack_ternary_kernel(
     const float *__restrict__ x, uint64_t n, float threshold, uint32_t *__restrict__ packed,
-    unsigned long long *__restrict__ survivors) {
+    uint64_t n_tiles, unsigned long long *__restrict__ survivors) {
+    __shared__ unsigned s_cnt[kBlock / 64];
     const uint64_t n_quads = (n + 3) / 4;
     const uint64_t n_words = (n + 15) / 16;
-    const uint64_t tile_quad0 = (uint64_t)blockIdx.x * (kBlock * 4);
-    float4 v[4];
-    bool full[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        uint64_t q = tile_quad0 + (uint64_t)j * kBlock + threadIdx.x;
-        full[j] = (q * 4 + 3) < n;
-        v[j] = full[j] ? reinterpret_cast<const float4 *>(x)[q] : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
     unsigned count = 0;
+    for (uint64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+        const uint64_t tile_quad0 = tile * (kBlock * 4);
+        float4 v[4];
+        bool full[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        uint64_t q = tile_quad0 + (uint64_t)j * kBlock + threadIdx.x;
-        uint32_t byte = 0;
-        if (full[j]) {
-            float e[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+        for (int j = 0; j < 4; ++j) {
+            uint64_t q = tile_quad0 + (uint64_t)j * kBlock + threadIdx.x;
+            full[j] = (q * 4 + 3) < n;
+            v[j] = full[j] ? reinterpret_cast<const float4 *>(x)[q]
+                           : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                byte |= ternary_code(e[i], threshold) << (2 * i);
-                count += fabsf(e[i]) > threshold ? 1u : 0u;
-            }
-        } else if (q < n_quads) {  // the single partial group at the tail
-            for (int i = 0; i < 4; ++i) {
-                uint64_t idx = q * 4 + i;
-                if (idx < n) {
-                    float e = x[idx];
-                    byte |= ternary_code(e, threshold) << (2 * i);
-                    count += fabsf(e) > threshold ? 1u : 0u;
+        for (int j = 0; j < 4; ++j) {
+            uint64_t q = tile_quad0 + (uint64_t)j * kBlock + threadIdx.x;
+            uint32_t byte = 0;
+            if (full[j]) {
+                float e[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    byte |= ternary_code(e[i], threshold) << (2 * i);
+                    count += fabsf(e[i]) > threshold ? 1u : 0u;
+                }
+            } else if (q < n_quads) {  // the single partial group at the tail
+                for (int i = 0; i < 4; ++i) {
+                    uint64_t idx = q * 4 + i;
+                    if (idx < n) {
+                        float e = x[idx];
+                        byte |= ternary_code(e, threshold) << (2 * i);
+                        count += fabsf(e) > threshold ? 1u : 0u;
+                    }
                 }
             }
+            uint32_t word = byte << (8 * (threadIdx.x & 3));
+            word |= __shfl_xor(word, 1);
+            word |= __shfl_xor(word, 2);
+            if ((threadIdx.x & 3) == 0 && (q >> 2) < n_words) packed[q >> 2] = word;
         }
-        uint32_t word = byte << (8 * (threadIdx.x & 3));
-        word |= __shfl_xor(word, 1);
-        word |= __shfl_xor(word, 2);
-        if ((threadIdx.x & 3) == 0 && (q >> 2) < n_words) packed[q >> 2] = word;
     }
     if (survivors) {
-        // wave sum, then one atomic per wave (integer: order does not matter)
+        // wave sum, block sum, then ONE atomic per workgroup (integer: order does not
+        // matter; thousands of atomics on one address would serialise in L2)
         for (int off = 32; off > 0; off >>= 1) count += __shfl_down(count, off);
-        if ((threadIdx.x & 63) == 0 && count) atomicAdd(survivors, (unsigned long long)count);
+        if ((threadIdx.x & 63) == 0) s_cnt[threadIdx.x >> 6] = count;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned long long t = 0;
+            for (int w = 0; w < kBlock / 64; ++w) t += s_cnt[w];
+            if (t) atomicAdd(survivors, t);
+        }
     }
 }
 
@@ -255,41 +266,109 @@ __global__ __launch_bounds__(1024) void seq_scan_kernel(const SeqMap *__restrict
     }
 }
 
-// Replays the crossing block with ordinary f32 additions (one wave; lane 0 adds).
-__global__ __launch_bounds__(64) void seq_replay_kernel(const float *__restrict__ x,
-                                                        uint64_t first, uint64_t n,
-                                                        uint32_t nblocks, int use_mask,
-                                                        float thr,
-                                                        SeqState *__restrict__ state) {
-    __shared__ float s_x[kSeqTile];
-    uint32_t es, k0;
-    seq_state_split(state->s_bits, &es, &k0);
+// Resolves the crossing block.  Its 256 chunks of 16 elements are mapped (one thread
+// each) and scanned from the state entering the block; the one chunk in which k reaches
+// 2^24 is replayed with ordinary f32 additions, which moves S into a new binade; the
+// chunks after it are mapped again for that binade, and so on to the end of the block.
+// Early blocks cross several binades (S doubles every few elements at first), later
+// ones at most one.
+__global__ __launch_bounds__(kBlock) void seq_replay_kernel(const float *__restrict__ x,
+                                                            uint64_t first, uint64_t n,
+                                                            uint32_t nblocks, int use_mask,
+                                                            float thr,
+                                                            SeqState *__restrict__ state) {
+    __shared__ SeqMap s_a[kBlock];
+    __shared__ SeqMap s_b[kBlock];
+    __shared__ unsigned s_first;
+    __shared__ uint32_t s_bits_now;
+    uint32_t es, k_cur;
+    seq_state_split(state->s_bits, &es, &k_cur);
     const uint32_t cb = state->cross_block;
+    const uint32_t t = threadIdx.x;
     if (cb == 0xffffffffu) {
-        if (threadIdx.x == 0) {
+        if (t == 0) {
             state->s_bits = seq_state_join(es, state->k);
             state->next_rel = nblocks;
         }
         return;
     }
-    const uint64_t base = first + (uint64_t)cb * kSeqTile;
-    for (int i = threadIdx.x; i < kSeqTile; i += 64) {
-        uint64_t idx = base + i;
-        float a = 0.0f;
-        bool take = false;
+    k_cur = state->k;
+    const uint64_t base = first + (uint64_t)cb * kSeqTile + (uint64_t)t * 16;
+    float a[16];
+    bool take[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint64_t idx = base + i;
+        float v = 0.0f;
+        bool tk = false;
         if (idx < n) {
-            a = fabsf(x[idx]);
-            take = use_mask ? (a > thr) : true;
+            v = fabsf(x[idx]);
+            tk = use_mask ? (v > thr) : true;
         }
         // a skipped element adds +0.0, which leaves any S >= 0 (and NaN/Inf) unchanged
-        s_x[i] = take ? a : 0.0f;
+        a[i] = tk ? v : 0.0f;
+        take[i] = tk;
     }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        float s = __uint_as_float(seq_state_join(es, state->k));
-#pragma unroll 8
-        for (int i = 0; i < kSeqTile; ++i) s = s + s_x[i];
-        state->s_bits = __float_as_uint(s);
+    uint32_t done = 0;  // chunks [0, done) are already folded into (es, k_cur)
+    uint32_t result_bits = 0;
+    for (int guard = 0; guard <= kBlock; ++guard) {
+        SeqMap m = seq_identity();
+        if (t >= done) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                if (take[i]) m = seq_append(m, __float_as_uint(a[i]), es);
+        }
+        if (t == 0) s_first = 0xffffffffu;
+        s_a[t] = m;
+        __syncthreads();
+        SeqMap *src = s_a, *dst = s_b;
+        for (uint32_t off = 1; off < (uint32_t)kBlock; off <<= 1) {
+            SeqMap v = src[t];
+            if (t >= off) v = seq_compose(src[t - off], v);
+            dst[t] = v;
+            __syncthreads();
+            SeqMap *tmp = src;
+            src = dst;
+            dst = tmp;
+        }
+        const SeqMap before = t == 0 ? seq_identity() : src[t - 1];
+        const uint32_t k = seq_apply(before, k_cur);
+        const bool crosses = t >= done && k < SEQ_K_LIMIT && seq_apply(m, k) >= SEQ_K_LIMIT;
+        if (crosses) atomicMin(&s_first, t);
+        const uint32_t k_end = seq_apply(src[kBlock - 1], k_cur);  // state after the block if no crossing
+        __syncthreads();
+        const uint32_t tstar = s_first;
+        if (tstar == 0xffffffffu) {
+            result_bits = seq_state_join(es, k_end);
+            break;
+        }
+        if (t == tstar) {
+            float sum = __uint_as_float(seq_state_join(es, k));
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sum = sum + a[i];
+            s_bits_now = __float_as_uint(sum);
+        }
+        __syncthreads();
+        result_bits = s_bits_now;
+        done = tstar + 1;
+        if (((result_bits >> 23) & 0xffu) == 0xffu) {
+            // S is +Inf or NaN.  +Inf turns into NaN if a NaN follows inside this block.
+            bool nan_after = false;
+            if (t >= done) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) nan_after |= (a[i] != a[i]);
+            }
+            if (nan_after) atomicOr(&s_bits_now, 0x7fc00000u);  // Inf | quiet bit = NaN
+            __syncthreads();
+            result_bits = s_bits_now;
+            break;
+        }
+        if (done >= (uint32_t)kBlock) break;
+        seq_state_split(result_bits, &es, &k_cur);
+        __syncthreads();  // s_first / s_bits_now are rewritten in the next turn
+    }
+    if (t == 0) {
+        state->s_bits = result_bits;
         state->next_rel = cb + 1;
     }
 }
@@ -404,7 +483,7 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     RBN_HIP(hipMemcpyAsync(&scr->seq, h_state, sizeof(SeqState), hipMemcpyHostToDevice,
                            ctx->stream));
     RBN_HIP(hipStreamSynchronize(ctx->stream));
-    uint64_t pos = 0;  // in blocks
+    uint64_t pos = 0;  // in blocks of kSeqTile elements
     uint32_t s_bits = 0;
     while (pos < total_blocks) {
         if (!is_finite_bits(s_bits)) break;
@@ -417,8 +496,8 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
         seq_block_maps_kernel<<<dim3((unsigned)win), dim3(kBlock), 0, ctx->stream>>>(
             d_x, first, n, es, use_mask, thr, maps);
         seq_scan_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(maps, (uint32_t)win, &scr->seq);
-        seq_replay_kernel<<<dim3(1), dim3(64), 0, ctx->stream>>>(d_x, first, n, (uint32_t)win,
-                                                                 use_mask, thr, &scr->seq);
+        seq_replay_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(d_x, first, n, (uint32_t)win,
+                                                                     use_mask, thr, &scr->seq);
         RBN_HIP(hipGetLastError());
         RBN_HIP(hipMemcpyAsync(h_state, &scr->seq, sizeof(SeqState), hipMemcpyDeviceToHost,
                                ctx->stream));
@@ -489,8 +568,9 @@ int pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold, ui
     }
     uint64_t tiles = (n + kSeqTile - 1) / kSeqTile;
     if (tiles > 0x7fffffffull) return rbn_fail(RBN_ERR_UNSUPPORTED, "tensor too large");
-    pack_ternary_kernel<<<dim3((unsigned)tiles), dim3(kBlock), 0, ctx->stream>>>(
-        d_x, n, threshold, (uint32_t *)d_packed, d_cnt);
+    const unsigned grid = (unsigned)(tiles < 8192 ? tiles : 8192);
+    pack_ternary_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
+        d_x, n, threshold, (uint32_t *)d_packed, tiles, d_cnt);
     RBN_HIP(hipGetLastError());
     if (h_survivors) {
         RBN_HIP(hipMemcpyAsync(ctx->mailbox, d_cnt, 8, hipMemcpyDeviceToHost, ctx->stream));
@@ -519,14 +599,13 @@ int rbn_abs_sum_f32(rbn_ctx *ctx, const float *d_x, uint64_t n, int mode, int us
     if (mode == RBN_SUM_TREE)
         return tree_abs_sum(ctx, d_x, n, use_mask, mask_threshold, h_sum, h_count);
     RBN_CHECK(strict_abs_sum(ctx, d_x, n, use_mask, mask_threshold, h_sum));
-    if (h_count) {
-        if (!use_mask) {
-            *h_count = n;
-        } else {
-            float unused;
-            RBN_CHECK(tree_abs_sum(ctx, d_x, n, 1, mask_threshold, &unused, h_count));
-        }
+    uint64_t count = n;
+    if (use_mask) {
+        float unused;
+        RBN_CHECK(tree_abs_sum(ctx, d_x, n, 1, mask_threshold, &unused, &count));
+        if (count == 0) *h_sum = -0.0f;  // the fold never ran: Rust's empty f32 sum
     }
+    if (h_count) *h_count = count;
     return RBN_OK;
 }
 

@@ -119,7 +119,7 @@ extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr
         return -0.0f;
     }
     const uint64_t total_blocks = (n + kTile - 1) / kTile;
-    uint64_t pos = 0;
+    uint64_t pos = 0;  // in blocks
     uint32_t s_bits = 0;
     while (pos < total_blocks) {
         if (((s_bits >> 23) & 0xff) == 0xff) break;
@@ -133,27 +133,71 @@ extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr
         for (uint64_t b = 0; b < win; ++b) maps[b] = block_map(x, first + b * kTile, n, es, use_mask, thr);
         read += win * kTile;
         ScanResult sr = scan(maps, s_bits);
-        uint32_t next_rel;
+        uint64_t next_rel;
         if (sr.cross_block == 0xffffffffu) {
             s_bits = seq_state_join(es, sr.k);
-            next_rel = (uint32_t)win;
+            next_rel = win;
         } else {
-            uint32_t jb = seq_state_join(es, sr.k);
-            float s;
-            std::memcpy(&s, &jb, 4);
-            uint64_t base = first + (uint64_t)sr.cross_block * kTile;
-            for (int i = 0; i < kTile; ++i) {
-                uint64_t idx = base + i;
-                float a = 0.0f;
-                bool take = false;
-                if (idx < n) {
-                    a = std::fabs(x[idx]);
-                    take = use_mask ? (a > thr) : true;
+            // the replay kernel: crossings inside the block are resolved one after another
+            const uint64_t bbase = first + (uint64_t)sr.cross_block * kTile;
+            uint32_t k_cur = sr.k, done = 0, result_bits = 0;
+            for (int guard = 0; guard <= 256; ++guard) {
+                SeqMap cm[256], a[256], b2[256];
+                for (int t = 0; t < 256; ++t)
+                    cm[t] = (uint32_t)t >= done ? thread_map(x, bbase + (uint64_t)t * 16, n, es, use_mask, thr)
+                                                : seq_identity();
+                for (int t = 0; t < 256; ++t) a[t] = cm[t];
+                SeqMap *src = a, *dst = b2;
+                for (int off = 1; off < 256; off <<= 1) {
+                    for (int t = 0; t < 256; ++t) {
+                        SeqMap v = src[t];
+                        if (t >= off) v = seq_compose(src[t - off], v);
+                        dst[t] = v;
+                    }
+                    std::swap(src, dst);
                 }
-                volatile float t = s + (take ? a : 0.0f);
-                s = t;
+                int tstar = -1;
+                uint32_t kstar = 0;
+                for (int t = 0; t < 256; ++t) {
+                    SeqMap before = t == 0 ? seq_identity() : src[t - 1];
+                    uint32_t kk = seq_apply(before, k_cur);
+                    if ((uint32_t)t >= done && kk < SEQ_K_LIMIT && seq_apply(cm[t], kk) >= SEQ_K_LIMIT) {
+                        tstar = t;
+                        kstar = kk;
+                        break;
+                    }
+                }
+                if (tstar < 0) {
+                    result_bits = seq_state_join(es, seq_apply(src[255], k_cur));
+                    break;
+                }
+                uint32_t jb = seq_state_join(es, kstar);
+                float s;
+                std::memcpy(&s, &jb, 4);
+                for (int i = 0; i < 16; ++i) {
+                    uint64_t idx = bbase + (uint64_t)tstar * 16 + i;
+                    float av = 0.0f;
+                    bool take = false;
+                    if (idx < n) {
+                        av = std::fabs(x[idx]);
+                        take = use_mask ? (av > thr) : true;
+                    }
+                    volatile float t2 = s + (take ? av : 0.0f);
+                    s = t2;
+                }
+                std::memcpy(&result_bits, &s, 4);
+                done = (uint32_t)tstar + 1;
+                if (((result_bits >> 23) & 0xff) == 0xff) {
+                    for (uint64_t idx = bbase + (uint64_t)done * 16; idx < bbase + kTile && idx < n; ++idx) {
+                        bool take = use_mask ? (std::fabs(x[idx]) > thr) : true;
+                        if (take && x[idx] != x[idx]) result_bits |= 0x7fc00000u;
+                    }
+                    break;
+                }
+                if (done >= 256) break;
+                seq_state_split(result_bits, &es, &k_cur);
             }
-            std::memcpy(&s_bits, &s, 4);
+            s_bits = result_bits;
             next_rel = sr.cross_block + 1;
         }
         pos += next_rel;
@@ -167,6 +211,13 @@ extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr
     }
     if (iterations) *iterations = iters;
     if (elements_read) *elements_read = read;
+    if (use_mask) {
+        // nothing survived the mask: the fold never ran and keeps Rust's initial -0.0
+        // (the device entry point knows this from the survivor count)
+        bool any = false;
+        for (uint64_t i = 0; i < n && !any; ++i) any = std::fabs(x[i]) > thr;
+        if (!any) return -0.0f;
+    }
     return s;
 }
 

@@ -1,0 +1,147 @@
+"""CPU-side checks: the C ABI loads and exports what the header declares, the host-only
+helpers follow the reference's size rules, the exact sequential-sum arithmetic that the
+HIP kernels share (ronn_amd/csrc/seqsum_core.h) reproduces a literal f32 fold, and the
+test helpers agree with the literal oracle.  No GPU work is launched here.
+"""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from ronn_amd import _lib
+from util import epilogue, exact_int_matmul
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_lib.LIB_PATH):
+        import __graft_entry__ as g
+        g.build()
+    return _lib.load()
+
+
+def test_library_exports_every_declared_symbol(lib):
+    header = open(os.path.join(ROOT, "include", "ronn_bitnet_hip.h")).read()
+    declared = set(re.findall(r"\b(rbn_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 35
+    for name in sorted(declared):
+        assert hasattr(lib, name), "%s is declared in the header but not exported" % name
+    # and the Python binding covers exactly the declared set
+    assert declared == set(_lib.SIGNATURES)
+
+
+def test_no_device_is_reported_not_faked(lib):
+    if lib.rbn_device_count() > 0:
+        pytest.skip("a GPU is visible here")
+    h = C.c_void_p()
+    rc = lib.rbn_ctx_create(0, C.byref(h))
+    assert rc == _lib.RBN_ERR_NO_DEVICE and h.value is None
+    assert b"no HIP device" in lib.rbn_last_error()
+    from ronn_amd.device import Context
+    with pytest.raises(_lib.RbnError):
+        Context(0)
+
+
+def test_size_rules_match_reference_allocator(lib):
+    # allocator.rs:231-235, :257-261, :285-288 and the oracle's restatement of :39-75
+    assert lib.rbn_tensor_bytes(1000, _lib.DT_BOOL) == 125
+    assert lib.rbn_tensor_bytes(100, _lib.DT_U8) == 25
+    assert lib.rbn_tensor_bytes(32 * 32, _lib.DT_BOOL) == 128
+    for dt in range(10):
+        for n in (0, 1, 3, 4, 5, 1000, 4097):
+            assert lib.rbn_tensor_bytes(n, dt) == O.packed_size([n], dt)
+        assert lib.rbn_tensor_alignment(dt) == O.alignment(dt)
+    assert lib.rbn_packed_capacity(100) >= 25 and lib.rbn_packed_capacity(100) % 16 == 0
+    assert lib.rbn_tiled_bytes(4096, 11008) == 4096 * 11008 // 4
+    assert lib.rbn_tiled_bytes(3, 2) == 64 * 64 // 4          # padded to 64 x 64
+    assert lib.rbn_act_pitch(2048) == 2048 and lib.rbn_act_pitch(100) == 128
+
+
+def test_synthetic_generator_is_deterministic_and_normal(lib):
+    from ronn_amd.device import synth_normal
+    a = synth_normal(7, 0.02, (100000,))
+    b = synth_normal(7, 0.02, (100000,))
+    assert (a == b).all()
+    # a range generated in two pieces equals the whole (counter-based)
+    c = np.concatenate([synth_normal(7, 0.02, (33333,)), synth_normal(7, 0.02, (66667,), first=33333)])
+    assert (a == c).all()
+    assert abs(float(a.mean())) < 3e-4 and abs(float(a.std()) - 0.02) < 2e-4
+    assert not (a == synth_normal(8, 0.02, (100000,))).any()
+
+
+@pytest.fixture(scope="module")
+def seqsum(tmp_path_factory):
+    out = str(tmp_path_factory.mktemp("seq") / "seqsum_host.so")
+    src = os.path.join(ROOT, "tests", "host", "seqsum_host.cpp")
+    subprocess.run(["g++", "-O2", "-ffp-contract=off", "-shared", "-fPIC", "-o", out, src], check=True)
+    L = C.CDLL(out)
+    L.seqsum_host.restype = C.c_float
+    L.seqsum_host.argtypes = [C.c_void_p, C.c_uint64, C.c_int, C.c_float, C.POINTER(C.c_uint64),
+                              C.POINTER(C.c_uint64)]
+    L.seqsum_literal.restype = C.c_float
+    L.seqsum_literal.argtypes = [C.c_void_p, C.c_uint64, C.c_int, C.c_float]
+    return L
+
+
+def _cases():
+    rng = np.random.default_rng(1)
+    yield "weights", rng.normal(0, 0.02, 4096 * 3 + 17)
+    yield "config1", rng.normal(0, 0.02, 2048 * 2048)
+    yield "acts", rng.normal(0, 1, 4096)
+    yield "zeros", np.zeros(10000)
+    yield "ones", np.full(100000, 1.0)
+    yield "ones_past_2^24", np.full((1 << 24) + 70000, 1.0)
+    yield "denormals", rng.normal(0, 1e-40, 100000)
+    yield "huge", rng.normal(0, 1e30, 100000)
+    yield "overflow", rng.normal(0, 3e37, 100000)
+    x = rng.normal(0, 1, 100000); x[5000] = np.inf
+    yield "inf", x
+    x = x.copy(); x[90000] = np.nan
+    yield "inf_then_nan", x
+    x = rng.normal(0, 1, 100000); x[5000] = np.inf; x[5100] = np.nan
+    yield "inf_then_nan_same_block", x
+    x = rng.normal(0, 1, 100000); x[70000] = np.nan
+    yield "nan", x
+    yield "lognormal", rng.lognormal(0, 6, 500000)
+    yield "cauchy", np.abs(rng.standard_cauchy(300000))
+    yield "ties_even", np.concatenate([[2.0 ** 20], np.full(300000, 2.0 ** -4)])
+    yield "ties_odd", np.concatenate([[2.0 ** 20 + 2.0 ** -3], np.full(300000, 2.0 ** -4)])
+    for n in (1, 2, 15, 16, 17, 4095, 4096, 4097):
+        yield "n%d" % n, rng.normal(0, 1, n)
+
+
+@pytest.mark.parametrize("name,x", list(_cases()), ids=lambda v: v if isinstance(v, str) else "")
+def test_parallel_sequential_sum_is_bit_exact(seqsum, name, x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    for mask, thr in ((0, 0.0), (1, float(np.median(np.abs(x[np.isfinite(x)]))) if x.size else 0.0)):
+        got = np.float32(seqsum.seqsum_host(x.ctypes.data, x.size, mask, thr, None, None))
+        want = np.float32(seqsum.seqsum_literal(x.ctypes.data, x.size, mask, thr))
+        assert got.view(np.uint32) == want.view(np.uint32) or (np.isnan(got) and np.isnan(want)), \
+            "%s mask=%d: %r vs %r" % (name, mask, got, want)
+
+
+def test_sequential_sum_traffic_is_bounded(seqsum):
+    # the window policy re-reads at most ~2x the data on the sizes that matter
+    x = np.random.default_rng(2).normal(0, 0.02, 4096 * 4096).astype(np.float32)
+    it, rd = C.c_uint64(), C.c_uint64()
+    seqsum.seqsum_host(x.ctypes.data, x.size, 0, 0.0, C.byref(it), C.byref(rd))
+    assert rd.value <= 2.0 * x.size and it.value <= 40
+
+
+def test_blas_helper_equals_literal_oracle_loop():
+    rng = np.random.default_rng(4)
+    for m, k, n in ((1, 300, 40), (5, 1000, 33), (16, 4096, 16)):
+        x = rng.normal(0, 1, (m, k)).astype(np.float32)
+        w = rng.normal(0, 0.02, (k, n)).astype(np.float32)
+        q, s, _ = O.act_quant_i8(x)
+        t = O.quantize_ternary(w)
+        out, acc = O.matmul_i8_ternary(q, s, t)
+        acc2 = exact_int_matmul(q, t.values().reshape(k, n))
+        assert (acc == acc2).all()
+        assert (out.view(np.uint32) == epilogue(acc2, s, t.scale).view(np.uint32)).all()

@@ -36,6 +36,24 @@ def test_library_exports_every_declared_symbol(lib):
     assert declared == set(_lib.SIGNATURES)
 
 
+def test_provider_abi_exports(lib):
+    from ronn_amd import bitnet
+    header = open(os.path.join(ROOT, "include", "ronn_bitnet_provider.h")).read()
+    declared = set(re.findall(r"\b(rbp_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 25
+    for name in sorted(declared):
+        assert hasattr(lib, name), "%s is declared in the header but not exported" % name
+    assert declared == set(bitnet.PROVIDER_SIGNATURES)
+
+
+def test_provider_without_device_raises(lib):
+    if lib.rbn_device_count() > 0:
+        pytest.skip("a GPU is visible here")
+    from ronn_amd import bitnet
+    with pytest.raises(bitnet.Error, match="no HIP device"):
+        bitnet.create_bitnet_provider()
+
+
 def test_no_device_is_reported_not_faked(lib):
     if lib.rbn_device_count() > 0:
         pytest.skip("a GPU is visible here")

@@ -144,6 +144,47 @@ def cpu_baseline(wl, out, acc, budget_s=20.0):
     return base, parity
 
 
+def profile_kernel(ctx, which, launches):
+    """Launches one kernel `launches` times on its real shape, for rocprofv3 runs.
+
+    gemv: M=1 K=4096 N=11008, rotating weight buffers.  gemm: M=2048 K=4096 N=11008.
+    pack / quantize: the 8192 x 28672 weight matrix of the large-layer config.
+    copy: a device-to-device copy of 256 MiB, whose known traffic calibrates the
+    FETCH_SIZE / WRITE_SIZE counters.
+    """
+    from ronn_amd import _lib
+    from ronn_amd.device import synth_normal
+    if which == "gemv":
+        wl = Workload(ctx, 1, 4096, 11008, 0.02, seed=2, mode=1)
+        for i in range(launches):
+            wl.launch(ctx.gemv, i)
+    elif which == "gemm":
+        wl = Workload(ctx, 2048, 4096, 11008, 0.02, seed=4, rotate_bytes=1, mode=1)
+        for i in range(launches):
+            wl.launch(ctx.gemm, 0)
+    elif which in ("pack", "quantize"):
+        K, N = 8192, 28672
+        d_w = ctx.alloc(4 * K * N)
+        rows = 512
+        for r0 in range(0, K, rows):   # generated and uploaded in slices to bound host memory
+            part = synth_normal(0x5EED1005, 0.015, (rows * N,), first=r0 * N)
+            _lib.check(ctx.lib.rbn_h2d(ctx.handle, d_w.ptr + 4 * r0 * N, part.ctypes.data, part.nbytes))
+        d_p = ctx.alloc(ctx.lib.rbn_packed_capacity(K * N))
+        for i in range(min(launches, 4)):
+            if which == "pack":
+                ctx.pack_ternary(d_w, K * N, 0.0028, d_p)
+            else:
+                ctx.quantize_ternary(d_w, K * N, _lib.SUM_STRICT_SEQ, d_p)
+    elif which == "copy":
+        n = 256 << 20
+        a, b = ctx.alloc(n), ctx.alloc(n)
+        _lib.check(ctx.lib.rbn_fill_u8(ctx.handle, a.ptr, 1, n))
+        for i in range(launches):
+            _lib.check(ctx.lib.rbn_d2d(ctx.handle, b.ptr, a.ptr, n))
+    ctx.sync()
+    print(json.dumps({"profiled_kernel": which, "launches": launches}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -151,6 +192,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=400)
     ap.add_argument("--no-extra", action="store_true", help="headline only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity gate")
+    ap.add_argument("--kernel", choices=["gemv", "gemm", "pack", "quantize", "copy"],
+                    help="profiling aid: launch only this kernel a few times (for rocprofv3) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); "
@@ -160,6 +203,9 @@ def main():
     from ronn_amd.device import Context
     ctx = Context(0)
     info = ctx.device_info()
+    if args.kernel:
+        profile_kernel(ctx, args.kernel, max(1, min(args.steps, 64)))
+        return
 
     M, K, N = 1, 4096, 11008
     wl = Workload(ctx, M, K, N, 0.02, seed=2, want_host=not args.no_cpu)

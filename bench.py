@@ -28,6 +28,9 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X published HBM3E bandwidth
 INT8_PEAK_TOPS = 5000.0     # MI355X published dense int8 MFMA rate (5.0 POP/s)
 MALL_BYTES = 256 << 20
+# HBM bytes per launch of the headline GEMV, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a
+# 256 MiB copy (profiles/gemv_m1_k4096_n11008.md)
+GEMV_HEADLINE_TRAFFIC_BYTES = 11424422
 
 
 def gemv_bytes(M, K, N):
@@ -229,7 +232,7 @@ def main():
                    "M": M, "K": K, "N": N, "device": info["name"], "arch": info["arch"],
                    "compute_units": info["compute_units"], "clock_mhz": info["clock_khz"] / 1000.0},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": GEMV_HEADLINE_TRAFFIC_BYTES,
                      "kernel": "gemv_t2_i8_kernel<1,8>", "bytes_per_launch": bytes_per_launch,
                      "us_per_launch": ev_ms * 1e3},
     }

@@ -33,7 +33,7 @@
  *             2-bit field at bit 8*b + 2*s (so (word >> 2*s) & 0x03030303 is four
  *             int8-ready codes of four consecutive k).  A quad's weights are thus
  *             contiguous along k.  Code = value + 1 (same as "packed"); 11 and padding
- *             are stored as 01 (zero).  Kpad = K rounded up to 64, Npad = N rounded up
+ *             are stored as 01 (zero).  Kpad = K rounded up to 128, Npad = N rounded up
  *             to 64.  Built from "packed" by rbn_tile_weights().
  */
 #ifndef RONN_BITNET_HIP_H
@@ -113,7 +113,7 @@ size_t rbn_tensor_alignment(int dtype);
 size_t rbn_packed_capacity(uint64_t n);
 /* Bytes of the "tiled" layout of a [K,N] weight matrix. */
 size_t rbn_tiled_bytes(uint64_t K, uint64_t N);
-/* Row pitch, in bytes, of quantised activations for inner dimension K (K rounded up to 64). */
+/* Row pitch, in bytes, of quantised activations for inner dimension K (K rounded up to 128). */
 size_t rbn_act_pitch(uint64_t K);
 
 /* ---- timing on the context's stream -------------------------------------- */

@@ -78,5 +78,5 @@ struct CtxGuard {
 static inline uint64_t round_up_u64(uint64_t v, uint64_t m) { return (v + m - 1) / m * m; }
 
 // Layout helpers (see the header for the formats).
-static inline uint64_t rbn_kpad(uint64_t K) { return round_up_u64(K, 64); }
+static inline uint64_t rbn_kpad(uint64_t K) { return round_up_u64(K, 128); }
 static inline uint64_t rbn_npad(uint64_t N) { return round_up_u64(N, 64); }

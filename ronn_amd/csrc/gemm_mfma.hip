@@ -5,36 +5,48 @@
 // crates/ronn-providers/src/bitnet/kernels.rs:134-178 (epilogue order :168).
 //
 // Shape of the kernel (v_mfma_i32_32x32x32_i8, 64-wide waves):
-//  * Workgroup tile 128 (M) x 256 (N), K step 128 per barrier; four waves as 2 x 2, each
-//    wave 64 x 128 = 2 x 4 MFMA tiles (128 accumulator registers), two workgroups per CU.
-//  * Weights stay 2-bit until they are in registers.  The tiled layout keeps the four
-//    columns of a quad in one 16-byte unit per 16 k, and a lane's B fragment for one MFMA
-//    (sixteen consecutive k of one column) is one u32 of it.  Lane l therefore reads ONE
-//    16-byte unit (quad l%32, k-half l/32) per K step of 32 and expands it with 28 VALU
-//    operations into the B fragments of FOUR MFMA tiles: tile j covers the columns
-//    4*quad + j.  The same mapping lets the epilogue store four adjacent columns per lane
-//    as one 128-bit store.
-//  * Both operands go through LDS, double-buffered: activations as int8 rows padded to
-//    144 B, weights still packed (2 KiB per 32 k) in [k-block][quad] order with an XOR
-//    swizzle so that the transposing store and the fragment loads are conflict-free.
-//    Global loads are whole 128-byte lines for both operands.
+//  * Workgroup tile 128 (M) x 256 (N), K step 128; four waves as 2 x 2, each wave
+//    64 x 128 = 2 x 4 MFMA tiles (128 accumulator registers), two workgroups per CU.
+//  * Both operands travel global memory -> LDS without touching registers
+//    (global_load_lds_dwordx4), into a ring of three stages: the loads of K step it+2 are
+//    issued while step it is multiplied, so HBM latency (each weight byte is used by only
+//    two row tiles per XCD and therefore misses L2) is covered by two K steps.  The loads
+//    are issued from inline assembly, so the compiler neither tracks nor waits for them;
+//    the ring is synchronised by hand: s_waitcnt vmcnt(6) leaves exactly the newest
+//    stage's six loads in flight, then a bare s_barrier.
+//  * A lane of such a load picks its own global address but lands at LDS base + 16 * lane,
+//    so the LDS images are linear arrays of 16-byte units with an XOR swizzle chosen so
+//    that (a) eight consecutive lanes fetch one 128-byte line of global memory and (b) the
+//    128-bit fragment reads of eight consecutive lanes hit distinct banks:
+//      activations  unit row*8 + (seg ^ (row & 7))   holds q[row][16*seg .. 16*seg+15]
+//      weights      unit quad*8 + (kb ^ (quad & 7))  holds the four words of (quad, kb)
+//  * Weights stay 2-bit until they are in registers.  Lane l reads ONE 16-byte unit (quad
+//    l%32, k-half l/32) per 32 k and expands it with 28 VALU operations into the B
+//    fragments of FOUR MFMA tiles: tile j covers the columns 4*quad + j.  The same mapping
+//    lets the epilogue store four adjacent columns per lane as one 128-bit store.
 //  * Workgroups are numbered so that the eight XCDs each own a band of rows: a band's
-//    activations (128 rows x K) stay in that XCD's L2 while the weights stream through.
+//    activations stay in that XCD's L2 while the weights stream through.
 //  * Weights are stored as code = value + 1, so the per-token sum of q is subtracted in
-//    the epilogue (integer-exact).
+//    the epilogue (integer-exact).  K is padded to 128 by the activation and weight
+//    formats (zero activations, zero-weight codes), rows and columns past the edge are
+//    clamped duplicates whose results are never stored.
 #include "common.hpp"
 
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef void __attribute__((address_space(3))) * lds_ptr;
+typedef const void __attribute__((address_space(1))) * global_ptr;
 
 constexpr int kThreads = 256;
 constexpr int BM = 128, BN = 256, BK = 128;
-constexpr int kARow = BK + 16;        // bytes per activation row in LDS
-constexpr int kQuads = BN / 4;        // 64 column quads per workgroup tile
-constexpr int kKb = BK / 16;          // 8 k-blocks per K step
-constexpr int kABytes = BM * kARow;   // 18432
+constexpr int kAUnits = BM * 8;        // 16-byte units of one activation stage (16 KiB)
+constexpr int kBUnits = (BN / 4) * 8;  // of one weight stage (8 KiB)
+
+// s_waitcnt immediates (gfx9 encoding: vmcnt[3:0] | expcnt << 4 | lgkmcnt << 8 | vmcnt[5:4] << 14)
+constexpr int kWaitVm6Lgkm0 = 0x0076;  // vmcnt(6) and lgkmcnt(0)
+constexpr int kWaitVm0 = 0x0F70;       // vmcnt(0)
 
 __device__ __forceinline__ v4i decode_b(uint32_t w) {
     v4i b;
@@ -45,23 +57,31 @@ __device__ __forceinline__ v4i decode_b(uint32_t w) {
     return b;
 }
 
-// 16-byte slot of (k-block kb, quad q) inside the packed weight tile in LDS
-__device__ __forceinline__ int b_slot(int kb, int q) { return kb * kQuads + (q ^ ((kb & 7) << 1)); }
+// One wave-wide 16-byte-per-lane load from global memory straight into LDS: lane i's
+// 16 bytes land at LDS byte address lds_wave_base + 16 * i (M0 carries the base).
+__device__ __forceinline__ void dma16(const void *src, uint32_t lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(lds_wave_base), "v"(src)
+                 : "memory", "m0");
+}
 
 __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
-    const int8_t *__restrict__ q,         // [M][Kpad]
+    const int8_t *__restrict__ q,         // [M][Kpad], Kpad % 128 == 0
     const float *__restrict__ act_scale,  // [M]
     const int32_t *__restrict__ rowsum,   // [M]
     const uint4 *__restrict__ wt,         // tiled: uint4 index quad * KB + kb
     float w_scale, int M, int Kpad, int N, int nquads, int m_tiles, int n_tiles,
     int32_t *__restrict__ acc_out, float *__restrict__ out) {
-    __shared__ __attribute__((aligned(16))) uint8_t s_a[2][kABytes];
-    __shared__ __attribute__((aligned(16))) uint4 s_b[2][kKb * kQuads];
+    // Ring of three stages in one array (units of 16 bytes): weights of stage s at
+    // s * kBUnits, activations at 3 * kBUnits + s * kAUnits.
+    __shared__ __attribute__((aligned(16))) uint4 smem[3 * (kAUnits + kBUnits)];
     __shared__ float s_scale[BM];
     __shared__ int s_rowsum[BM];
 
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     const int KB = Kpad >> 4;
 
@@ -94,84 +114,62 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    // staging assignments: A tile 128 rows x 128 B = 1024 units of 16 B (4 per thread);
-    // B tile 64 quads x 8 k-blocks = 512 units (2 per thread)
-    const int a_seg = tid & 7, a_row0 = tid >> 3;      // rows a_row0 + 32*j
-    const int b_kb = tid & 7, b_q0 = tid >> 3;         // quads b_q0 + 32*j
-    uint4 ra[4], rb[2];
-    // Loads are unconditional (clamped addresses) and their results are not touched until
-    // store_tiles(), after the MFMA section: anything that consumes a loaded register
-    // earlier would make the compiler wait for the load in front of the matrix work.
-    auto load_tiles = [&](int k0) {
-        const int kb0 = k0 >> 4;
+    // Per-lane source addresses of the stage loads.  Load j of wave w fills the units
+    // (4j + w) * 64 + lane: row (or quad) (4j + w) * 8 + lane / 8, slot lane % 8, and the
+    // slot holds segment (or k-block) slot ^ (row & 7) = (lane & 7) ^ (lane >> 3).
+    const int sub = lane >> 3, slot_src = (lane & 7) ^ (lane >> 3);
+    const int8_t *a_src[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int row = m0 + a_row0 + 32 * j;
-            const int k = k0 + a_seg * 16;
-            ra[j] = *reinterpret_cast<const uint4 *>(q + (size_t)min(row, M - 1) * Kpad +
-                                                     min(k, Kpad - 16));
-        }
+    for (int j = 0; j < 4; ++j) {
+        const int row = min(m0 + (4 * j + wave) * 8 + sub, M - 1);
+        a_src[j] = q + (size_t)row * Kpad + slot_src * 16;
+    }
+    const uint4 *b_src[2];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int quad = q0 + b_q0 + 32 * j;
-            const int kb = kb0 + b_kb;
-            rb[j] = wt[(size_t)min(quad, nquads - 1) * KB + min(kb, KB - 1)];
-        }
-    };
-    // Out-of-range rows / k contribute zero activations; out-of-range columns / k get the
-    // zero-weight code.
-    auto store_tiles = [&](int buf, int k0) {
-        const int kb0 = k0 >> 4;
+    for (int j = 0; j < 2; ++j) {
+        const int quad = min(q0 + (4 * j + wave) * 8 + sub, nquads - 1);
+        b_src[j] = wt + (size_t)quad * KB + slot_src;
+    }
+    const int iters = Kpad / BK;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr)smem;
+    auto issue = [&](int it, int stage) {
+        const int kk = min(it, iters - 1);  // past the end: reload the last step, never read
+        const uint32_t sb = lds0 + (uint32_t)(stage * kBUnits) * 16;
+        const uint32_t sa = lds0 + (uint32_t)(3 * kBUnits + stage * kAUnits) * 16;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int row = m0 + a_row0 + 32 * j;
-            const int k = k0 + a_seg * 16;
-            const uint32_t keep = (row < M && k < Kpad) ? 0xffffffffu : 0u;
-            *reinterpret_cast<uint4 *>(&s_a[buf][(a_row0 + 32 * j) * kARow + a_seg * 16]) =
-                make_uint4(ra[j].x & keep, ra[j].y & keep, ra[j].z & keep, ra[j].w & keep);
-        }
+        for (int j = 0; j < 4; ++j) dma16(a_src[j] + (size_t)kk * BK, sa + (4 * j + wave) * 1024);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int quad = q0 + b_q0 + 32 * j;
-            const bool ok = quad < nquads && kb0 + b_kb < KB;
-            s_b[buf][b_slot(b_kb, b_q0 + 32 * j)] =
-                make_uint4(ok ? rb[j].x : 0x55555555u, ok ? rb[j].y : 0x55555555u,
-                           ok ? rb[j].z : 0x55555555u, ok ? rb[j].w : 0x55555555u);
-        }
+        for (int j = 0; j < 2; ++j)
+            dma16(b_src[j] + (size_t)kk * (BK / 16), sb + (4 * j + wave) * 1024);
     };
 
-    load_tiles(0);
-    store_tiles(0, 0);
-    __syncthreads();
+    // fragment addresses (in 16-byte units, relative to a stage)
+    const int frow0 = wm * 64 + (lane & 31), khalf = lane >> 5;
+    const int fquad = wn * 32 + (lane & 31);
+    auto a_unit = [&](int row, int seg) { return row * 8 + (seg ^ (row & 7)); };
+    auto b_unit = [&](int kb) { return fquad * 8 + (kb ^ (fquad & 7)); };
 
-    const int iters = (Kpad + BK - 1) / BK;
-    const int a_lane_off = (lane & 31) * kARow + (lane >> 5) * 16;
-    for (int it = 0; it < iters; ++it) {
-        const int cur = it & 1;
-        const bool more = it + 1 < iters;
-        if (more) load_tiles((it + 1) * BK);
-        __builtin_amdgcn_sched_barrier(0);
-        // Fragments of K step ks+1 are fetched from LDS while the MFMAs of step ks run.
-        uint4 bw = s_b[cur][b_slot(lane >> 5, wn * 32 + (lane & 31))];
-        v4i af0 = *reinterpret_cast<const v4i *>(&s_a[cur][(wm * 64) * kARow + a_lane_off]);
-        v4i af1 = *reinterpret_cast<const v4i *>(&s_a[cur][(wm * 64 + 32) * kARow + a_lane_off]);
+    auto multiply = [&](int stage) {
+        const uint4 *sb = smem + stage * kBUnits;
+        const uint4 *sa = smem + 3 * kBUnits + stage * kAUnits;
+        uint4 bw = sb[b_unit(khalf)];
+        uint4 a0 = sa[a_unit(frow0, khalf)];
+        uint4 a1 = sa[a_unit(frow0 + 32, khalf)];
 #pragma unroll
         for (int ks = 0; ks < BK / 32; ++ks) {
-            uint4 bw_n = bw;
-            v4i af0_n = af0, af1_n = af1;
-            if (ks + 1 < BK / 32) {
-                bw_n = s_b[cur][b_slot((ks + 1) * 2 + (lane >> 5), wn * 32 + (lane & 31))];
-                af0_n = *reinterpret_cast<const v4i *>(
-                    &s_a[cur][(wm * 64) * kARow + a_lane_off + (ks + 1) * 32]);
-                af1_n = *reinterpret_cast<const v4i *>(
-                    &s_a[cur][(wm * 64 + 32) * kARow + a_lane_off + (ks + 1) * 32]);
+            uint4 bw_n = bw, a0_n = a0, a1_n = a1;
+            if (ks + 1 < BK / 32) {  // next sub-step's fragments, fetched under this one's MFMAs
+                bw_n = sb[b_unit((ks + 1) * 2 + khalf)];
+                a0_n = sa[a_unit(frow0, (ks + 1) * 2 + khalf)];
+                a1_n = sa[a_unit(frow0 + 32, (ks + 1) * 2 + khalf)];
             }
-            // B: one 16-byte unit per lane -> fragments of the four column tiles
             v4i bf[4];
             bf[0] = decode_b(bw.x);
             bf[1] = decode_b(bw.y);
             bf[2] = decode_b(bw.z);
             bf[3] = decode_b(bw.w);
+            const v4i af0 = {(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w};
+            const v4i af1 = {(int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 acc[0][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af0, bf[j], acc[0][j], 0, 0, 0);
@@ -179,17 +177,36 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
             for (int j = 0; j < 4; ++j)
                 acc[1][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af1, bf[j], acc[1][j], 0, 0, 0);
             bw = bw_n;
-            af0 = af0_n;
-            af1 = af1_n;
+            a0 = a0_n;
+            a1 = a1_n;
         }
-        __builtin_amdgcn_sched_barrier(0);
-        if (more) store_tiles(cur ^ 1, (it + 1) * BK);
-        __syncthreads();
+    };
+
+    // prologue: stages 0 and 1 in flight, wait for stage 0 (and for the LDS writes above)
+    issue(0, 0);
+    issue(1, 1);
+    __builtin_amdgcn_s_waitcnt(kWaitVm6Lgkm0);
+    __builtin_amdgcn_s_barrier();
+
+    // One K step on stage `cur`: start the loads of step it+2 into `fill` (the stage read in
+    // step it-1, which every wave has left: it passed the barrier that ended that step),
+    // multiply, then wait until only those newest six loads are outstanding and meet.
+    int cur = 0, fill = 2;
+    for (int it = 0; it < iters; ++it) {
+        issue(it + 2, fill);
+        multiply(cur);
+        // lgkmcnt(0) too: this wave's own LDS reads of `cur` must have returned before any
+        // wave may start overwriting that stage in the next step
+        __builtin_amdgcn_s_waitcnt(kWaitVm6Lgkm0);
+        __builtin_amdgcn_s_barrier();
+        cur = cur == 2 ? 0 : cur + 1;
+        fill = fill == 2 ? 0 : fill + 1;
     }
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);  // no load may still be writing LDS at exit
 
     // epilogue: lane owns columns 4*quad .. 4*quad+3 (tile j -> column 4*quad + j) and rows
     // 8*(r/4) + 4*(lane/32) + r%4 of each 32-row tile
-    const int col0 = n0 + (wn * 32 + (lane & 31)) * 4;
+    const int col0 = n0 + fquad * 4;
     const bool vec_ok = (N & 3) == 0;
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt) {
@@ -241,6 +258,7 @@ extern "C" int rbn_gemm_t2_i8_mfma(rbn_ctx *ctx, const int8_t *d_q, const float 
                 "d_out and d_acc must be 16-byte aligned");
     RBN_REQUIRE(M <= (1ull << 24) && K <= (1ull << 24) && N <= (1ull << 24), "dimension too large");
     const int Kpad = (int)rbn_kpad(K);
+    static_assert(BK == 128, "the K padding of the formats must equal the K step");
     const int nquads = (int)(rbn_npad(N) / 4);
     const int m_tiles = (int)((M + BM - 1) / BM), n_tiles = (int)((N + BN - 1) / BN);
     const uint64_t tiles = (uint64_t)m_tiles * n_tiles;

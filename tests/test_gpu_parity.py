@@ -190,7 +190,7 @@ def test_tile_weights(ctx, K, N):
 def test_tile_weights_sanitises_invalid_code(ctx):
     raw = np.full(64 * 64 // 4, 0xFF, dtype=np.uint8)     # every field is 11
     d_t = ctx.tile_weights(ctx.to_device(raw), 64, 64)
-    assert (decode_tiled(d_t.download(np.uint32, 64 * 64 // 16), 64, 64) == 0).all()
+    assert (decode_tiled(d_t.download(np.uint32, ctx.lib.rbn_tiled_bytes(64, 64) // 4), 64, 64) == 0).all()
 
 
 # ---- (2) activation quantisation -----------------------------------------------------------
@@ -215,7 +215,7 @@ def test_act_quant_i8_ties_and_extremes(ctx):
                   [-127.0, 126.5, -126.5, 125.5, 0.49999997, -0.0, 1e-30, -1e-30]], dtype=np.float32)
     q, s, rs = O.act_quant_i8(x)
     d_q, d_s, d_r = ctx.act_quant_i8(ctx.to_device(x), 2, 8)
-    got = d_q.download(np.int8, 2 * 64).reshape(2, 64)[:, :8]
+    got = d_q.download(np.int8, 2 * ctx.act_pitch(8)).reshape(2, ctx.act_pitch(8))[:, :8]
     assert (got == q).all() and q[0].tolist() == [127, 0, 2, 2, 0, -2, -2, 3]
     assert same_bits(d_s.download(np.float32, 2), s)
 

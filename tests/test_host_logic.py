@@ -77,7 +77,7 @@ def test_size_rules_match_reference_allocator(lib):
         assert lib.rbn_tensor_alignment(dt) == O.alignment(dt)
     assert lib.rbn_packed_capacity(100) >= 25 and lib.rbn_packed_capacity(100) % 16 == 0
     assert lib.rbn_tiled_bytes(4096, 11008) == 4096 * 11008 // 4
-    assert lib.rbn_tiled_bytes(3, 2) == 64 * 64 // 4          # padded to 64 x 64
+    assert lib.rbn_tiled_bytes(3, 2) == 128 * 64 // 4         # padded to 128 x 64
     assert lib.rbn_act_pitch(2048) == 2048 and lib.rbn_act_pitch(100) == 128
 
 

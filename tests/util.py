@@ -44,7 +44,7 @@ def decode_tiled(tiled_words, K, N):
     Word ((q * KB + kb) * 4 + c) belongs to column 4q+c and k-block kb; inside a word the
     weight k = 16*kb + 4*s + b sits at bit 8*b + 2*s as code = value + 1.
     """
-    kpad = (K + 63) // 64 * 64
+    kpad = (K + 127) // 128 * 128
     npad = (N + 63) // 64 * 64
     kb_n = kpad // 16
     t = np.asarray(tiled_words, dtype=np.uint32).reshape(npad // 4, kb_n, 4)

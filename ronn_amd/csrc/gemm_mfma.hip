@@ -18,8 +18,11 @@
 //    so the LDS images are linear arrays of 16-byte units with an XOR swizzle chosen so
 //    that (a) eight consecutive lanes fetch one 128-byte line of global memory and (b) the
 //    128-bit fragment reads of eight consecutive lanes hit distinct banks:
-//      activations  unit row*8 + (seg ^ (row & 7))   holds q[row][16*seg .. 16*seg+15]
-//      weights      unit quad*8 + (kb ^ (quad & 7))  holds the four words of (quad, kb)
+//      activations  unit row*8 + (seg ^ ((row>>1) & 7))   holds q[row][16*seg .. 16*seg+15]
+//      weights      unit quad*8 + (kb ^ ((quad>>1) & 7))  holds the four words of (quad, kb)
+//    (LDS serves sixteen lanes of a 128-bit read per cycle from 64 banks: sixteen
+//    consecutive rows must fall on sixteen different 16-byte bank groups, i.e. distinct
+//    values of (row & 1) * 8 + slot, which the (row >> 1) swizzle gives)
 //  * Weights stay 2-bit until they are in registers.  Lane l reads ONE 16-byte unit (quad
 //    l%32, k-half l/32) per 32 k and expands it with 28 VALU operations into the B
 //    fragments of FOUR MFMA tiles: tile j covers the columns 4*quad + j.  The same mapping
@@ -116,19 +119,21 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
 
     // Per-lane source addresses of the stage loads.  Load j of wave w fills the units
     // (4j + w) * 64 + lane: row (or quad) (4j + w) * 8 + lane / 8, slot lane % 8, and the
-    // slot holds segment (or k-block) slot ^ (row & 7) = (lane & 7) ^ (lane >> 3).
-    const int sub = lane >> 3, slot_src = (lane & 7) ^ (lane >> 3);
+    // slot holds segment (or k-block) slot ^ ((row >> 1) & 7) of that row.
+    const int sub = lane >> 3;
     const int8_t *a_src[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-        const int row = min(m0 + (4 * j + wave) * 8 + sub, M - 1);
-        a_src[j] = q + (size_t)row * Kpad + slot_src * 16;
+        const int lrow = (4 * j + wave) * 8 + sub;
+        const int seg = (lane & 7) ^ ((lrow >> 1) & 7);
+        a_src[j] = q + (size_t)min(m0 + lrow, M - 1) * Kpad + seg * 16;
     }
     const uint4 *b_src[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const int quad = min(q0 + (4 * j + wave) * 8 + sub, nquads - 1);
-        b_src[j] = wt + (size_t)quad * KB + slot_src;
+        const int lquad = (4 * j + wave) * 8 + sub;
+        const int kb = (lane & 7) ^ ((lquad >> 1) & 7);
+        b_src[j] = wt + (size_t)min(q0 + lquad, nquads - 1) * KB + kb;
     }
     const int iters = Kpad / BK;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr)smem;
@@ -146,39 +151,62 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
     // fragment addresses (in 16-byte units, relative to a stage)
     const int frow0 = wm * 64 + (lane & 31), khalf = lane >> 5;
     const int fquad = wn * 32 + (lane & 31);
-    auto a_unit = [&](int row, int seg) { return row * 8 + (seg ^ (row & 7)); };
-    auto b_unit = [&](int kb) { return fquad * 8 + (kb ^ (fquad & 7)); };
+    auto a_unit = [&](int row, int seg) { return row * 8 + (seg ^ ((row >> 1) & 7)); };
+    auto b_unit = [&](int kb) { return fquad * 8 + (kb ^ ((fquad >> 1) & 7)); };
 
+    // One K step (four sub-steps of 32 k) as a software pipeline inside the wave:
+    //   sub-step ks multiplies with fragments that are already decoded, while the VALU
+    //   expands the weights of ks+1 and LDS delivers the raw fragments of ks+2.
+    // A v_mfma_i32_32x32x32_i8 holds the matrix pipe for 32 cycles, during which the wave
+    // can issue about seven other instructions; sched_group_barrier asks the scheduler for
+    // exactly that interleaving (1 MFMA, a few VALU, sometimes one LDS read) instead of
+    // "all expansion, then all MFMAs".
     auto multiply = [&](int stage) {
         const uint4 *sb = smem + stage * kBUnits;
         const uint4 *sa = smem + 3 * kBUnits + stage * kAUnits;
-        uint4 bw = sb[b_unit(khalf)];
-        uint4 a0 = sa[a_unit(frow0, khalf)];
-        uint4 a1 = sa[a_unit(frow0 + 32, khalf)];
+        constexpr int S = BK / 32;
+        uint4 braw[S], a0raw[S], a1raw[S];
+        braw[0] = sb[b_unit(khalf)];
+        a0raw[0] = sa[a_unit(frow0, khalf)];
+        a1raw[0] = sa[a_unit(frow0 + 32, khalf)];
+        braw[1] = sb[b_unit(2 + khalf)];
+        a0raw[1] = sa[a_unit(frow0, 2 + khalf)];
+        a1raw[1] = sa[a_unit(frow0 + 32, 2 + khalf)];
+        v4i bf[4], bf_n[4];
+        bf[0] = decode_b(braw[0].x);
+        bf[1] = decode_b(braw[0].y);
+        bf[2] = decode_b(braw[0].z);
+        bf[3] = decode_b(braw[0].w);
 #pragma unroll
-        for (int ks = 0; ks < BK / 32; ++ks) {
-            uint4 bw_n = bw, a0_n = a0, a1_n = a1;
-            if (ks + 1 < BK / 32) {  // next sub-step's fragments, fetched under this one's MFMAs
-                bw_n = sb[b_unit((ks + 1) * 2 + khalf)];
-                a0_n = sa[a_unit(frow0, (ks + 1) * 2 + khalf)];
-                a1_n = sa[a_unit(frow0 + 32, (ks + 1) * 2 + khalf)];
+        for (int ks = 0; ks < S; ++ks) {
+            if (ks + 2 < S) {
+                braw[ks + 2] = sb[b_unit((ks + 2) * 2 + khalf)];
+                a0raw[ks + 2] = sa[a_unit(frow0, (ks + 2) * 2 + khalf)];
+                a1raw[ks + 2] = sa[a_unit(frow0 + 32, (ks + 2) * 2 + khalf)];
             }
-            v4i bf[4];
-            bf[0] = decode_b(bw.x);
-            bf[1] = decode_b(bw.y);
-            bf[2] = decode_b(bw.z);
-            bf[3] = decode_b(bw.w);
-            const v4i af0 = {(int)a0.x, (int)a0.y, (int)a0.z, (int)a0.w};
-            const v4i af1 = {(int)a1.x, (int)a1.y, (int)a1.z, (int)a1.w};
+            if (ks + 1 < S) {
+                bf_n[0] = decode_b(braw[ks + 1].x);
+                bf_n[1] = decode_b(braw[ks + 1].y);
+                bf_n[2] = decode_b(braw[ks + 1].z);
+                bf_n[3] = decode_b(braw[ks + 1].w);
+            }
+            const v4i af0 = {(int)a0raw[ks].x, (int)a0raw[ks].y, (int)a0raw[ks].z, (int)a0raw[ks].w};
+            const v4i af1 = {(int)a1raw[ks].x, (int)a1raw[ks].y, (int)a1raw[ks].z, (int)a1raw[ks].w};
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 acc[0][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af0, bf[j], acc[0][j], 0, 0, 0);
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 acc[1][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af1, bf[j], acc[1][j], 0, 0, 0);
-            bw = bw_n;
-            a0 = a0_n;
-            a1 = a1_n;
+            // interleave: 8 x (1 MFMA + 4 VALU), the first three groups also take an LDS read
+#pragma unroll
+            for (int g = 0; g < 8; ++g) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+                if (g < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+                __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // VALU
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bf[j] = bf_n[j];
         }
     };
 

@@ -154,81 +154,100 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
     auto a_unit = [&](int row, int seg) { return row * 8 + (seg ^ ((row >> 1) & 7)); };
     auto b_unit = [&](int kb) { return fquad * 8 + (kb ^ ((fquad >> 1) & 7)); };
 
-    // One K step (four sub-steps of 32 k) as a software pipeline inside the wave:
-    //   sub-step ks multiplies with fragments that are already decoded, while the VALU
-    //   expands the weights of ks+1 and LDS delivers the raw fragments of ks+2.
-    // A v_mfma_i32_32x32x32_i8 holds the matrix pipe for 32 cycles, during which the wave
-    // can issue about seven other instructions; sched_group_barrier asks the scheduler for
-    // exactly that interleaving (1 MFMA, a few VALU, sometimes one LDS read) instead of
-    // "all expansion, then all MFMAs".
-    auto multiply = [&](int stage) {
+    // Lane-constant fragment offsets (16-byte units inside a stage) of the four sub-steps.
+    int a_off[4], b_off[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        a_off[ks] = a_unit(frow0, 2 * ks + khalf);
+        b_off[ks] = b_unit(2 * ks + khalf);
+    }
+
+    // The K loop is a software pipeline that spans the stage boundary.  A K step has four
+    // sub-steps of 32 k; sub-step ks multiplies with fragments that are already in
+    // registers (weights decoded), while the VALU expands the weights of the next sub-step
+    // and LDS delivers the raw fragments of the sub-step after that - across the boundary
+    // the "next" sub-steps are sub-steps 0 and 1 of the following stage.  The stage
+    // hand-over (wait for the DMA, barrier) therefore sits in the MIDDLE of a K step,
+    // between sub-steps 1 and 2: by then every read of the current stage has been issued
+    // (and is waited for), and the reads of the next stage start right after it, a full
+    // sub-step (eight MFMAs, 256 cycles) before their first use.
+    // A v_mfma_i32_32x32x32_i8 holds the matrix pipe for 32 cycles, in which the wave can
+    // issue about seven other instructions; sched_group_barrier asks for that interleaving
+    // (1 MFMA + 4 VALU, the first three groups also an LDS read), and sched_barrier(0)
+    // keeps the compiler from moving anything between sub-steps (left alone it sinks every
+    // LDS read down to its first use and waits for it there).
+    uint4 rb[4], ra0[4], ra1[4];
+    v4i bf[4], bf_n[4];
+    auto lds_reads = [&](int stage, int ks) {
         const uint4 *sb = smem + stage * kBUnits;
         const uint4 *sa = smem + 3 * kBUnits + stage * kAUnits;
-        constexpr int S = BK / 32;
-        uint4 braw[S], a0raw[S], a1raw[S];
-        braw[0] = sb[b_unit(khalf)];
-        a0raw[0] = sa[a_unit(frow0, khalf)];
-        a1raw[0] = sa[a_unit(frow0 + 32, khalf)];
-        braw[1] = sb[b_unit(2 + khalf)];
-        a0raw[1] = sa[a_unit(frow0, 2 + khalf)];
-        a1raw[1] = sa[a_unit(frow0 + 32, 2 + khalf)];
-        v4i bf[4], bf_n[4];
-        bf[0] = decode_b(braw[0].x);
-        bf[1] = decode_b(braw[0].y);
-        bf[2] = decode_b(braw[0].z);
-        bf[3] = decode_b(braw[0].w);
+        rb[ks] = sb[b_off[ks]];
+        ra0[ks] = sa[a_off[ks]];
+        ra1[ks] = sa[a_off[ks] + 32 * 8];  // row + 32: same swizzle
+    };
+    auto decode_next = [&](int ks) {
+        bf_n[0] = decode_b(rb[ks].x);
+        bf_n[1] = decode_b(rb[ks].y);
+        bf_n[2] = decode_b(rb[ks].z);
+        bf_n[3] = decode_b(rb[ks].w);
+    };
+    // sub-step ks: read (read_stage, read_ks), decode dec_ks, multiply ks
+    auto substep = [&](int ks, int read_stage, int read_ks, int dec_ks) {
+        lds_reads(read_stage, read_ks);
+        decode_next(dec_ks);
+        const v4i af0 = {(int)ra0[ks].x, (int)ra0[ks].y, (int)ra0[ks].z, (int)ra0[ks].w};
+        const v4i af1 = {(int)ra1[ks].x, (int)ra1[ks].y, (int)ra1[ks].z, (int)ra1[ks].w};
 #pragma unroll
-        for (int ks = 0; ks < S; ++ks) {
-            if (ks + 2 < S) {
-                braw[ks + 2] = sb[b_unit((ks + 2) * 2 + khalf)];
-                a0raw[ks + 2] = sa[a_unit(frow0, (ks + 2) * 2 + khalf)];
-                a1raw[ks + 2] = sa[a_unit(frow0 + 32, (ks + 2) * 2 + khalf)];
-            }
-            if (ks + 1 < S) {
-                bf_n[0] = decode_b(braw[ks + 1].x);
-                bf_n[1] = decode_b(braw[ks + 1].y);
-                bf_n[2] = decode_b(braw[ks + 1].z);
-                bf_n[3] = decode_b(braw[ks + 1].w);
-            }
-            const v4i af0 = {(int)a0raw[ks].x, (int)a0raw[ks].y, (int)a0raw[ks].z, (int)a0raw[ks].w};
-            const v4i af1 = {(int)a1raw[ks].x, (int)a1raw[ks].y, (int)a1raw[ks].z, (int)a1raw[ks].w};
+        for (int j = 0; j < 4; ++j)
+            acc[0][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af0, bf[j], acc[0][j], 0, 0, 0);
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[0][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af0, bf[j], acc[0][j], 0, 0, 0);
+        for (int j = 0; j < 4; ++j)
+            acc[1][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af1, bf[j], acc[1][j], 0, 0, 0);
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                acc[1][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af1, bf[j], acc[1][j], 0, 0, 0);
-            // interleave: 8 x (1 MFMA + 4 VALU), the first three groups also take an LDS read
-#pragma unroll
-            for (int g = 0; g < 8; ++g) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-                if (g < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-                __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // VALU
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) bf[j] = bf_n[j];
+        for (int g = 0; g < 8; ++g) {
+            if (g < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // MFMA
+            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);             // VALU
         }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bf[j] = bf_n[j];
+        __builtin_amdgcn_sched_barrier(0);
     };
 
-    // prologue: stages 0 and 1 in flight, wait for stage 0 (and for the LDS writes above)
+    // prologue: stages 0 and 1 in flight, wait for stage 0 (and for the LDS writes above),
+    // then fill the pipeline: raw fragments of sub-steps 0 and 1, weights of 0 decoded
     issue(0, 0);
     issue(1, 1);
     __builtin_amdgcn_s_waitcnt(kWaitVm6Lgkm0);
     __builtin_amdgcn_s_barrier();
+    lds_reads(0, 0);
+    lds_reads(0, 1);
+    decode_next(0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) bf[j] = bf_n[j];
+    __builtin_amdgcn_sched_barrier(0);
 
-    // One K step on stage `cur`: start the loads of step it+2 into `fill` (the stage read in
-    // step it-1, which every wave has left: it passed the barrier that ended that step),
-    // multiply, then wait until only those newest six loads are outstanding and meet.
-    int cur = 0, fill = 2;
+    // K step `it` on stage cur: start the loads of step it+2 into `fill` - the stage read
+    // in step it-1, which every wave has left: all its reads were waited for before the
+    // barrier inside step it-1.  After sub-step 1, wait until only those newest six loads
+    // are outstanding (stage nxt has landed) and until this wave's reads of `cur` have
+    // returned, meet, and go on with the reads of nxt.  In the last step nxt holds no
+    // new data; what is read from it is never used.
+    int cur = 0, nxt = 1, fill = 2;
     for (int it = 0; it < iters; ++it) {
         issue(it + 2, fill);
-        multiply(cur);
-        // lgkmcnt(0) too: this wave's own LDS reads of `cur` must have returned before any
-        // wave may start overwriting that stage in the next step
+        __builtin_amdgcn_sched_barrier(0);
+        substep(0, cur, 2, 1);
+        substep(1, cur, 3, 2);
         __builtin_amdgcn_s_waitcnt(kWaitVm6Lgkm0);
         __builtin_amdgcn_s_barrier();
-        cur = cur == 2 ? 0 : cur + 1;
-        fill = fill == 2 ? 0 : fill + 1;
+        __builtin_amdgcn_sched_barrier(0);
+        substep(2, nxt, 0, 3);
+        substep(3, nxt, 1, 0);
+        const int t = cur;
+        cur = nxt;
+        nxt = fill;
+        fill = t;
     }
     __builtin_amdgcn_s_waitcnt(kWaitVm0);  // no load may still be writing LDS at exit
 

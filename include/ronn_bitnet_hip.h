@@ -186,12 +186,19 @@ int rbn_act_quant_ternary(rbn_ctx *ctx, const float *d_x, uint64_t M, uint64_t K
 /* out[m,n] = ((float)acc[m,n] * act_scale[m]) * w_scale, acc = sum_k q[m,k]*w[k,n]
  * in int32.  d_acc may be NULL; when given it receives the int32 accumulators.
  * rbn_gemv_t2_i8: decode regime (M <= RBN_GEMV_MAX_M), streams the tiled weights
- * once with int8 dot instructions.  rbn_gemm_t2_i8_mfma: prefill regime, int8 MFMA.
- * rbn_matmul_t2_i8 picks one by M. */
+ * once with int8 dot instructions.  rbn_gemm_t2_i8_skinny: small batches
+ * (M <= RBN_SKINNY_MAX_M), the same streaming read with 16x16x64 int8 MFMA doing
+ * the dot products.  rbn_gemm_t2_i8_mfma: prefill regime, 128x256 tiles of int8
+ * MFMA.  rbn_matmul_t2_i8 picks one by M (1..3: gemv, 4..64: skinny, above: mfma).
+ * All three give identical results. */
 #define RBN_GEMV_MAX_M 16
+#define RBN_SKINNY_MAX_M 64
 int rbn_gemv_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
                    const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale, uint64_t M,
                    uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);
+int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
+                          const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
+                          uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);
 int rbn_gemm_t2_i8_mfma(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
                         const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
                         uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);

@@ -91,7 +91,10 @@ int rbn_ctx_create(int device, rbn_ctx **out) {
     if ((e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking)) != hipSuccess ||
         (e = hipEventCreate(&ctx->ev_start)) != hipSuccess ||
         (e = hipEventCreate(&ctx->ev_stop)) != hipSuccess ||
-        (e = hipHostMalloc(&ctx->mailbox, 4096, hipHostMallocDefault)) != hipSuccess) {
+        (e = hipHostMalloc(&ctx->mailbox, 4096, hipHostMallocDefault)) != hipSuccess ||
+        (e = hipMalloc(&ctx->splitk_partials, (size_t)RBN_SPLITK_TILES * 4096)) != hipSuccess ||
+        (e = hipMalloc((void **)&ctx->splitk_tickets, RBN_SPLITK_GROUPS * sizeof(unsigned))) != hipSuccess ||
+        (e = hipMemset(ctx->splitk_tickets, 0, RBN_SPLITK_GROUPS * sizeof(unsigned))) != hipSuccess) {
         int rc = rbn_fail(RBN_ERR_HIP, "context set-up failed: %s", hipGetErrorString(e));
         rbn_ctx_destroy(ctx);
         return rc;
@@ -106,6 +109,8 @@ int rbn_ctx_destroy(rbn_ctx *ctx) {
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->ws) (void)hipFree(ctx->ws);
     if (ctx->mailbox) (void)hipHostFree(ctx->mailbox);
+    if (ctx->splitk_partials) (void)hipFree(ctx->splitk_partials);
+    if (ctx->splitk_tickets) (void)hipFree(ctx->splitk_tickets);
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
     if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);

@@ -321,9 +321,13 @@ extern "C" int rbn_matmul_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_
                                 const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
                                 uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc,
                                 float *d_out) {
-    if (M <= RBN_GEMV_MAX_M)
+    // measured crossover: the dot-instruction GEMV wins up to three tokens
+    if (M <= 3)
         return rbn_gemv_t2_i8(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N, d_acc,
                               d_out);
+    if (M <= RBN_SKINNY_MAX_M)
+        return rbn_gemm_t2_i8_skinny(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N,
+                                     d_acc, d_out);
     return rbn_gemm_t2_i8_mfma(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N, d_acc,
                                d_out);
 }

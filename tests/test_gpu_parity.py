@@ -306,6 +306,60 @@ def test_gemm_mfma_small(ctx, M, K, N):
     check_against_oracle(x, w, *res, literal=(M * K * N <= 1 << 23))
 
 
+@pytest.mark.parametrize("M", [1, 2, 3, 7, 16, 17, 31, 32, 33, 48, 64])
+@pytest.mark.parametrize("K,N", [(64, 64), (128, 64), (2048, 2048), (100, 37), (4096, 96), (130, 1376),
+                                 (1100, 130)])
+def test_skinny_small_literal(ctx, M, K, N):
+    say("skinny", M, K, N)
+    x = synth_normal(0x5EED0005 + M, 1.0, (M, K))
+    w = synth_normal(0x5EED1005 + K, 0.02, (K, N))
+    res = run_matmul(ctx, ctx.skinny, x, w)
+    check_against_oracle(x, w, *res, literal=(M * K * N <= 1 << 23))
+
+
+@pytest.mark.parametrize("M", [4, 16, 64])
+@pytest.mark.parametrize("K,N", [(4096, 4096), (4096, 11008), (11008, 4096), (8192, 28672)])
+def test_skinny_sweep_shapes(ctx, M, K, N):
+    # decode sweep and the large-layer shape; the expected integers come through BLAS
+    if (K, N) == (8192, 28672):
+        if M == 16:
+            pytest.skip("the large-layer shape runs at M = 8 and 64")
+        M = 8 if M == 4 else M
+    say("skinny sweep", M, K, N)
+    x = synth_normal(0x5EED0006 + M, 1.0, (M, K))
+    w = synth_normal(0x5EED1006 + N, 0.015 if K == 8192 else 0.02, (K, N))
+    res = run_matmul(ctx, ctx.skinny, x, w)
+    check_against_oracle(x, w, *res, literal=False)
+
+
+def test_skinny_saturated_activations(ctx):
+    M, K, N = 48, 8192, 128
+    x = np.where(synth_normal(7, 1.0, (M, K)) > 0, 1.0, -1.0).astype(np.float32)
+    w = np.where(synth_normal(8, 1.0, (K, N)) > 0, 1.0, -1.0).astype(np.float32)
+    res = run_matmul(ctx, ctx.skinny, x, w)
+    check_against_oracle(x, w, *res, literal=False)
+    assert np.abs(res[1]).max() > 127 * 100
+
+
+@pytest.mark.parametrize("M", [1, 2, 16, 17, 64, 65, 128])
+def test_matmul_dispatch_agrees_across_kernels(ctx, M):
+    # rbn_matmul_t2_i8 picks gemv / skinny / mfma by M; every kernel that accepts the shape
+    # must return the same bits
+    K, N = 1024, 520
+    x = synth_normal(0x5EED0007 + M, 1.0, (M, K))
+    w = synth_normal(0x5EED1007, 0.02, (K, N))
+    ref = run_matmul(ctx, ctx.matmul, x, w)
+    check_against_oracle(x, w, *ref, literal=False)
+    fns = [ctx.gemm]
+    if M <= 16:
+        fns.append(ctx.gemv)
+    if M <= 64:
+        fns.append(ctx.skinny)
+    for fn in fns:
+        got = run_matmul(ctx, fn, x, w)
+        assert (got[1] == ref[1]).all() and same_bits(got[0], ref[0])
+
+
 def test_gemm_mfma_saturated_activations(ctx):
     # every activation at +-127/-128 and dense +-1 weights: the largest |acc| the path can see
     M, K, N = 64, 4096, 128
@@ -332,6 +386,9 @@ def test_error_paths(ctx):
     with pytest.raises(_lib.RbnError) as e:
         ctx.gemv((d, d, d), d, 1.0, 17, 64, 64)
     assert e.value.code == _lib.RBN_ERR_INVALID and "M <= 16" in e.value.message
+    with pytest.raises(_lib.RbnError) as e:
+        ctx.skinny((d, d, d), d, 1.0, 65, 64, 64)
+    assert e.value.code == _lib.RBN_ERR_INVALID and "M <= 64" in e.value.message
     with pytest.raises(_lib.RbnError):
         ctx.gemv((d, d, d), d, 1.0, 0, 64, 64)
     rc = ctx.lib.rbn_quantize_ternary(ctx.handle, d.ptr + 4, 16, 0, d.ptr, None, None, None)

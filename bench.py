@@ -81,7 +81,10 @@ class Workload:
 
 def time_graph(ctx, wl, fn, steps, warmup):
     """Average milliseconds per launch over `steps` launches replayed from a HIP graph."""
-    per_graph = len(wl.tiled)
+    # at least 32 launches per graph replay, so that the cost of launching the graph itself
+    # (several microseconds) does not hide the kernel; a whole number of buffer rotations
+    nbuf = len(wl.tiled)
+    per_graph = nbuf * max(1, -(-32 // nbuf))
     ctx.graph_begin()
     for i in range(per_graph):
         wl.launch(fn, i)
@@ -111,6 +114,41 @@ def time_plain(ctx, fn_call, reps):
         fn_call()
     ms = ctx.timer_stop()
     return ms / reps
+
+
+def time_ternarize(ctx, K, N, sigma):
+    """Absmean ternarisation + 2-bit packing of a K x N f32 matrix resident in HBM.
+
+    strict: the reference's sequential f32 sums reproduced exactly (bit-exact threshold and
+    scale); tree: pairwise sums (same packed bytes unless the threshold's last bit differs).
+    Algorithmic bytes: the matrix is read for the threshold sum, for the survivor sum and
+    for packing (3 x 4 n) and n / 4 bytes are written.
+    """
+    from ronn_amd import _lib
+    from ronn_amd.device import synth_normal
+    n = K * N
+    d_w = ctx.alloc(4 * n)
+    rows = 512
+    for r0 in range(0, K, rows):   # generated and uploaded in slices to bound host memory
+        part = synth_normal(0x5EED1005, sigma, (rows * N,), first=r0 * N)
+        _lib.check(ctx.lib.rbn_h2d(ctx.handle, d_w.ptr + 4 * r0 * N, part.ctypes.data, part.nbytes))
+    d_p = ctx.alloc(ctx.lib.rbn_packed_capacity(n))
+    out = {"K": K, "N": N, "weights": n}
+    for name, mode in (("strict", _lib.SUM_STRICT_SEQ), ("tree", _lib.SUM_TREE)):
+        ctx.quantize_ternary(d_w, n, mode, d_p)
+        ctx.sync()
+        t0 = time.perf_counter()
+        reps = 3
+        for _ in range(reps):
+            ctx.quantize_ternary(d_w, n, mode, d_p)
+        ctx.sync()
+        ms = (time.perf_counter() - t0) * 1e3 / reps
+        b = 3 * 4 * n + n // 4
+        out[name] = {"ms": ms, "Gweights_per_s": n / ms / 1e6, "GBps": b / ms / 1e6,
+                     "frac_hbm_peak": b / ms / 1e6 / HBM_PEAK_GBS}
+    d_w.free()
+    d_p.free()
+    return out
 
 
 def cpu_baseline(wl, out, acc, budget_s=20.0):
@@ -256,24 +294,38 @@ def main():
                                     "GBps": bytes_per_launch / (ev1 * 1e-3) / 1e9,
                                     "note": "single 11 MiB weight buffer re-read from cache, not HBM"}
         del one
-        sweep = []
-        for (k, n) in ((4096, 4096), (4096, 11008), (11008, 4096)):
-            for m in (1, 4, 16):
-                w2 = wl if (m, k, n) == (M, K, N) else Workload(ctx, m, k, n, 0.02, seed=3, mode=1)
-                ev, _, _ = time_graph(ctx, w2, ctx.gemv, 1500, 150)
-                b = gemv_bytes(m, k, n)
-                sweep.append({"M": m, "K": k, "N": n, "us": ev * 1e3, "GBps": b / (ev * 1e-3) / 1e9,
-                              "frac_hbm_peak": b / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS})
-                if w2 is not wl:
-                    del w2
-        extra["decode_sweep"] = sweep
+        def kernel_for(m):
+            return "gemv" if m <= 3 else ("skinny_mfma" if m <= 64 else "gemm_mfma")
+
+        def sweep_over(shapes, ms, sigma):
+            rows = []
+            for (k, n) in shapes:
+                for m in ms:
+                    w2 = wl if (m, k, n) == (M, K, N) else Workload(ctx, m, k, n, sigma, seed=3, mode=1)
+                    ev, _, _ = time_graph(ctx, w2, ctx.matmul, 1500, 150)
+                    b = gemv_bytes(m, k, n)
+                    rows.append({"M": m, "K": k, "N": n, "kernel": kernel_for(m), "us": ev * 1e3,
+                                 "GBps": b / (ev * 1e-3) / 1e9,
+                                 "frac_hbm_peak": b / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS})
+                    if w2 is not wl:
+                        del w2
+            return rows
+
+        # rbn_matmul_t2_i8 picks the kernel by M; weights rotate through > 256 MiB of buffers
+        extra["decode_sweep"] = sweep_over(((4096, 4096), (4096, 11008), (11008, 4096)), (1, 4, 16), 0.02)
+        extra["large_layer"] = sweep_over(((8192, 28672),), (1, 8, 64), 0.015)
+        extra["large_layer_ternarize"] = time_ternarize(ctx, 8192, 28672, 0.015)
         # prefill GEMM, int8 MFMA
         pm, pk, pn = 2048, 4096, 11008
         pw = Workload(ctx, pm, pk, pn, 0.02, seed=4, rotate_bytes=1, mode=1)
         ms = time_plain(ctx, lambda: pw.launch(ctx.gemm, 0), 20)
         ops = 2.0 * pm * pk * pn
         extra["prefill_gemm"] = {"M": pm, "K": pk, "N": pn, "ms": ms, "TOPS": ops / (ms * 1e-3) / 1e12,
-                                 "frac_int8_peak": ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS}
+                                 "frac_int8_peak": ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS,
+                                 "roofline": {"bound": "mfma", "achieved": ops / (ms * 1e-3) / 1e12,
+                                              "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                                              "frac": ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS,
+                                              "kernel": "gemm_t2_i8_mfma_kernel"}}
         del pw
         result["extra"] = extra
 

@@ -121,8 +121,8 @@ def time_ternarize(ctx, K, N, sigma):
 
     strict: the reference's sequential f32 sums reproduced exactly (bit-exact threshold and
     scale); tree: pairwise sums (same packed bytes unless the threshold's last bit differs).
-    Algorithmic bytes: the matrix is read for the threshold sum, for the survivor sum and
-    for packing (3 x 4 n) and n / 4 bytes are written.
+    Algorithmic bytes: 2 x 4 n + n / 4 (two reads are inherent: the threshold depends on
+    the global mean; the survivor sum can ride on the packing pass).
     """
     from ronn_amd import _lib
     from ronn_amd.device import synth_normal
@@ -143,7 +143,7 @@ def time_ternarize(ctx, K, N, sigma):
             ctx.quantize_ternary(d_w, n, mode, d_p)
         ctx.sync()
         ms = (time.perf_counter() - t0) * 1e3 / reps
-        b = 3 * 4 * n + n // 4
+        b = 2 * 4 * n + n // 4
         out[name] = {"ms": ms, "Gweights_per_s": n / ms / 1e6, "GBps": b / ms / 1e6,
                      "frac_hbm_peak": b / ms / 1e6 / HBM_PEAK_GBS}
     d_w.free()
@@ -188,7 +188,8 @@ def cpu_baseline(wl, out, acc, budget_s=20.0):
 def profile_kernel(ctx, which, launches):
     """Launches one kernel `launches` times on its real shape, for rocprofv3 runs.
 
-    gemv: M=1 K=4096 N=11008, rotating weight buffers.  gemm: M=2048 K=4096 N=11008.
+    gemv: M=1 K=4096 N=11008, rotating weight buffers.  skinny: M=16, same matrix.
+    gemm: M=2048 K=4096 N=11008.
     pack / quantize: the 8192 x 28672 weight matrix of the large-layer config.
     copy: a device-to-device copy of 256 MiB, whose known traffic calibrates the
     FETCH_SIZE / WRITE_SIZE counters.
@@ -199,6 +200,10 @@ def profile_kernel(ctx, which, launches):
         wl = Workload(ctx, 1, 4096, 11008, 0.02, seed=2, mode=1)
         for i in range(launches):
             wl.launch(ctx.gemv, i)
+    elif which == "skinny":
+        wl = Workload(ctx, 16, 4096, 11008, 0.02, seed=3, mode=1)
+        for i in range(launches):
+            wl.launch(ctx.skinny, i)
     elif which == "gemm":
         wl = Workload(ctx, 2048, 4096, 11008, 0.02, seed=4, rotate_bytes=1, mode=1)
         for i in range(launches):
@@ -233,7 +238,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=400)
     ap.add_argument("--no-extra", action="store_true", help="headline only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity gate")
-    ap.add_argument("--kernel", choices=["gemv", "gemm", "pack", "quantize", "copy"],
+    ap.add_argument("--kernel", choices=["gemv", "skinny", "gemm", "pack", "quantize", "copy"],
                     help="profiling aid: launch only this kernel a few times (for rocprofv3) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -327,6 +332,10 @@ def main():
                                               "frac": ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS,
                                               "kernel": "gemm_t2_i8_mfma_kernel"}}
         del pw
+        # what a loop of nothing but int8 MFMA sustains on this box, by operand values
+        extra["mfma_i8_probe_TOPS"] = {"constant_operands": ctx.probe_mfma_i8(0),
+                                       "int8_x_ternary_codes": ctx.probe_mfma_i8(1),
+                                       "int8_x_int8": ctx.probe_mfma_i8(2)}
         result["extra"] = extra
 
     print(json.dumps(result))

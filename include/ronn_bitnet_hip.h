@@ -214,6 +214,18 @@ int rbn_matmul_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
 int rbn_execute_ternary_matmul(rbn_ctx *ctx, const float *h_a, const float *h_b, uint64_t M,
                                uint64_t N, uint64_t K, int mode, float *h_out, int32_t *h_acc);
 
+/* ---- calibration probe (no reference counterpart) -------------------------- */
+/* Runs a loop of nothing but v_mfma_i32_32x32x32_i8 on every SIMD (operands in
+ * registers) and returns the dense int8 rate in TOP/s: the ceiling a GEMM on this
+ * machine can be priced against besides the published 5.0 POP/s.  The sustained
+ * clock depends on the operand values; operand_kind picks them. */
+enum rbn_probe_operands {
+    RBN_PROBE_CONSTANT = 0,   /* every byte 1 */
+    RBN_PROBE_I8_TERNARY = 1, /* random int8 x ternary codes {0,1,2}: this path's data */
+    RBN_PROBE_I8_I8 = 2       /* random int8 x random int8 */
+};
+int rbn_probe_mfma_i8(rbn_ctx *ctx, int operand_kind, double *h_tops);
+
 /* ---- synthetic inputs (host) ----------------------------------------------- */
 /* out[i] = (float)(sigma * z_i), z_i standard normal from a counter-based
  * generator: two 24-bit uniforms from splitmix64(seed, i/2), Box-Muller in

@@ -219,6 +219,12 @@ class Context:
         return self._mm(self.lib.rbn_matmul_t2_i8, acts, d_tiled, w_scale, M, K, N, want_acc,
                         d_out, d_acc)
 
+    def probe_mfma_i8(self, operand_kind: int) -> float:
+        """Dense int8 MFMA rate of this machine in TOP/s (0 constant, 1 int8 x ternary, 2 int8 x int8)."""
+        tops = C.c_double()
+        check(self.lib.rbn_probe_mfma_i8(self.handle, operand_kind, C.byref(tops)))
+        return tops.value
+
     # -- whole execute() -------------------------------------------------------------------
     def execute_ternary_matmul(self, a: np.ndarray, b: np.ndarray, mode=_lib.SUM_STRICT_SEQ,
                                want_acc=True):

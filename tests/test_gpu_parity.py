@@ -396,3 +396,11 @@ def test_error_paths(ctx):
     rc = ctx.lib.rbn_gemv_t2_i8(ctx.handle, None, None, None, None, 1.0, 1, 64, 64, None, None)
     assert rc == _lib.RBN_ERR_INVALID and b"null pointer" in ctx.lib.rbn_last_error()
     assert ctx.lib.rbn_sync(None) == _lib.RBN_ERR_INVALID
+
+
+def test_mfma_probe_reports_a_plausible_rate(ctx):
+    const = ctx.probe_mfma_i8(0)
+    tern = ctx.probe_mfma_i8(1)
+    assert 1000 < tern <= const * 1.05 < 5500
+    with pytest.raises(_lib.RbnError):
+        ctx.probe_mfma_i8(7)

@@ -214,6 +214,44 @@ int rbn_matmul_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
 int rbn_execute_ternary_matmul(rbn_ctx *ctx, const float *h_a, const float *h_b, uint64_t M,
                                uint64_t N, uint64_t K, int mode, float *h_out, int32_t *h_acc);
 
+/* ---- decoder building blocks (no reference counterpart) --------------------- */
+/* The reference's BitNet provider stops at the matmul; these are the usual
+ * LLaMA / BitNet-b1.58 operations a decoder needs around it, so that a whole decode
+ * step runs on the device and can be captured in a graph (positions and tokens are
+ * read from device memory).  All row-major f32 unless said otherwise. */
+/* x[m,:] = table[tokens[m],:] (token ids clamped to [0, vocab)). */
+int rbn_embed_f32(rbn_ctx *ctx, const float *d_table, const int32_t *d_tokens, uint64_t M,
+                  uint64_t H, uint64_t vocab, float *d_x);
+/* If d_delta: x += delta, written back (residual stream).  Then
+ * y = (x * rsqrt(mean(x^2) + eps)) * gamma, quantised per token exactly as
+ * rbn_act_quant_i8 does (same output format).  H <= 8192. */
+int rbn_rmsnorm_quant_i8(rbn_ctx *ctx, float *d_x, const float *d_delta, const float *d_gamma,
+                         float eps, uint64_t M, uint64_t H, int8_t *d_q, float *d_act_scale,
+                         int32_t *d_rowsum);
+/* d_qkv [M, 3*heads*head_dim] = (q | k | v).  Rotary embedding (pairs
+ * (i, i + head_dim/2), angle pos * theta^(-2i/head_dim), pos = *d_pos0 + m) of q in
+ * place and of k on its way into the cache: rotated k and v go to the f16 caches
+ * [heads][max_seq][head_dim] at pos; k and v in d_qkv stay as they were. */
+int rbn_rope_kv_store_f16(rbn_ctx *ctx, float *d_qkv, const int32_t *d_pos0, uint64_t M,
+                          uint64_t heads, uint64_t head_dim, float theta, void *d_kcache,
+                          void *d_vcache, uint64_t max_seq);
+/* Causal softmax(q.k / sqrt(head_dim)).v of token m over cache positions
+ * 0 .. *d_pos0 + m; head_dim must be 128.  d_out [M, heads*head_dim]. */
+int rbn_attention_f16kv(rbn_ctx *ctx, const float *d_qkv, const int32_t *d_pos0, uint64_t M,
+                        uint64_t heads, uint64_t head_dim, const void *d_kcache,
+                        const void *d_vcache, uint64_t max_seq, float *d_out);
+/* h[m,f] = silu(gu[m,f]) * gu[m,F+f], gu [M, 2F]. */
+int rbn_swiglu_f32(rbn_ctx *ctx, const float *d_gate_up, uint64_t M, uint64_t F, float *d_h);
+/* *d_index = index of the largest value (lowest index among equals).  If d_history
+ * is given the index is also written to d_history[*d_history_pos]. */
+int rbn_argmax_f32(rbn_ctx *ctx, const float *d_values, uint64_t n, int32_t *d_index,
+                   int32_t *d_history, const int32_t *d_history_pos);
+/* *d_value += delta (the position counter of a captured decode step). */
+int rbn_add_i32(rbn_ctx *ctx, int32_t *d_value, int32_t delta);
+/* Normal(0, sigma) values generated on the device (counter-based, f32 Box-Muller);
+ * for random-initialised weights; not the generator of rbn_synth_normal_f32. */
+int rbn_synth_normal_device_f32(rbn_ctx *ctx, uint64_t seed, float sigma, float *d_out, uint64_t n);
+
 /* ---- calibration probe (no reference counterpart) -------------------------- */
 /* Runs a loop of nothing but v_mfma_i32_32x32x32_i8 on every SIMD (operands in
  * registers) and returns the dense int8 rate in TOP/s: the ceiling a GEMM on this

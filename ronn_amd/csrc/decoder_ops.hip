@@ -1,0 +1,420 @@
+// Building blocks of a BitNet-style decoder around the ternary matmuls: embedding lookup,
+// RMSNorm fused with the per-token int8 quantisation (and the residual add), rotary
+// embedding + f16 K/V cache store, attention over the f16 cache, SwiGLU, arg-max.
+//
+// None of this exists in the reference (crates/ronn-providers/src/bitnet/ holds only the
+// quantiser, the matmul kernels and the provider); the formulas are the usual LLaMA /
+// BitNet-b1.58 ones and are pinned by the numpy model in tests/decoder_model.py.
+// Everything is stream-ordered and takes the current position from device memory, so a
+// whole decode step can be captured once in a HIP graph and replayed.
+#include <hip/hip_fp16.h>
+
+#include "common.hpp"
+
+namespace {
+
+constexpr int kBlock = 256;
+
+__device__ __forceinline__ float wave_sum_f(float v) {
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+__device__ __forceinline__ float wave_max_f(float v) {
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+// x[m, :] = table[tokens[m], :]
+__global__ __launch_bounds__(kBlock) void embed_kernel(const float *__restrict__ table,
+                                                       const int32_t *__restrict__ tokens, int H,
+                                                       int vocab, float *__restrict__ x) {
+    const int m = blockIdx.x;
+    int tok = tokens[m];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+    const float *src = table + (size_t)tok * H;
+    for (int i = threadIdx.x; i < H; i += kBlock) x[(size_t)m * H + i] = src[i];
+}
+
+// One workgroup per token:
+//   if delta: x += delta (written back: the residual stream)
+//   y = x * rsqrt(mean(x^2) + eps) * gamma
+//   g = max(max|y|, 1e-5); q = clamp(rne(y * (127/g)), -128, 127); scale = g/127; rowsum = sum q
+// The row (H <= kBlock * kPer floats) stays in registers between the passes.
+constexpr int kPer = 32;  // H <= 8192
+__global__ __launch_bounds__(kBlock) void rmsnorm_quant_kernel(
+    float *__restrict__ x, const float *__restrict__ delta, const float *__restrict__ gamma,
+    float eps, int H, int pitch, int8_t *__restrict__ q, float *__restrict__ act_scale,
+    int32_t *__restrict__ rowsum) {
+    __shared__ float s_red[kBlock / 64];
+    __shared__ int s_redi[kBlock / 64];
+    const int m = blockIdx.x, tid = threadIdx.x;
+    float *row = x + (size_t)m * H;
+    const float *drow = delta ? delta + (size_t)m * H : nullptr;
+    float v[kPer];
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        const int i = tid + j * kBlock;
+        float t = 0.0f;
+        if (i < H) {
+            t = row[i];
+            if (drow) {
+                t += drow[i];
+                row[i] = t;
+            }
+        }
+        v[j] = t;
+        ss += t * t;
+    }
+    ss = wave_sum_f(ss);
+    if ((tid & 63) == 0) s_red[tid >> 6] = ss;
+    __syncthreads();
+    ss = (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
+    const float inv_rms = 1.0f / sqrtf(ss / (float)H + eps);
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        const int i = tid + j * kBlock;
+        const float y = i < H ? (v[j] * inv_rms) * gamma[i] : 0.0f;
+        v[j] = y;
+        amax = fmaxf(amax, fabsf(y));
+    }
+    amax = wave_max_f(amax);
+    __syncthreads();
+    if ((tid & 63) == 0) s_red[tid >> 6] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    const float gmax = fmaxf(amax, 1e-5f);
+    const float inv = 127.0f / gmax;
+    int sum = 0;
+    int8_t *qrow = q + (size_t)m * pitch;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+        const int i = tid + j * kBlock;
+        if (i < pitch) {
+            float r = rintf(v[j] * inv);  // round half to even; 0 in the padding
+            r = fminf(fmaxf(r, -128.0f), 127.0f);
+            const int qi = i < H ? (int)r : 0;
+            qrow[i] = (int8_t)qi;
+            sum += qi;
+        }
+    }
+    sum = wave_sum_i(sum);
+    if ((tid & 63) == 0) s_redi[tid >> 6] = sum;
+    __syncthreads();
+    if (tid == 0) {
+        act_scale[m] = gmax / 127.0f;
+        rowsum[m] = (s_redi[0] + s_redi[1]) + (s_redi[2] + s_redi[3]);
+    }
+}
+
+// qkv: [M][3 * heads * hd] f32 (q | k | v).  Rotates q in place by the angle
+// pos * theta^(-2i/hd) on the pairs (i, i + hd/2), rotates k the same way on its way into
+// the cache, and stores k and v as f16 at position pos = *pos0 + m of the caches
+// [heads][max_seq][hd].
+__global__ __launch_bounds__(kBlock) void rope_kv_store_kernel(
+    float *__restrict__ qkv, const int32_t *__restrict__ pos0, int heads, int hd, float theta,
+    __half *__restrict__ kcache, __half *__restrict__ vcache, int max_seq) {
+    const int m = blockIdx.x;
+    const int pos = pos0[0] + m;
+    const int HD = heads * hd, half = hd >> 1;
+    float *qrow = qkv + (size_t)m * 3 * HD;
+    for (int idx = threadIdx.x; idx < heads * half; idx += kBlock) {
+        const int h = idx / half, i = idx - h * half;
+        const float freq = powf(theta, -2.0f * (float)i / (float)hd);
+        float sn, cs;
+        sincosf((float)pos * freq, &sn, &cs);
+        float *qh = qrow + h * hd, *kh = qrow + HD + h * hd;
+        const float *vh = qrow + 2 * HD + h * hd;
+        const float q0 = qh[i], q1 = qh[i + half];
+        qh[i] = q0 * cs - q1 * sn;
+        qh[i + half] = q1 * cs + q0 * sn;
+        const float k0 = kh[i], k1 = kh[i + half];
+        const float r0 = k0 * cs - k1 * sn, r1 = k1 * cs + k0 * sn;
+        if (pos < max_seq) {
+            const size_t c = ((size_t)h * max_seq + pos) * hd;
+            kcache[c + i] = __float2half_rn(r0);
+            kcache[c + i + half] = __float2half_rn(r1);
+            vcache[c + i] = __float2half_rn(vh[i]);
+            vcache[c + i + half] = __float2half_rn(vh[i + half]);
+        }
+    }
+}
+
+// Attention of token m (position p = *pos0 + m) and head h over cache positions 0..p.
+// One workgroup per (m, h); hd == 128.  Each wave takes every kWaves-th block of 64 keys:
+// scores with one key per lane (the key row is read as 16 x 16 bytes), online softmax,
+// then P.V with two dimensions per lane; the waves' (max, sum, out) meet through LDS.
+template <int kWaves>
+__global__ __launch_bounds__(kWaves * 64) void attention_kernel(
+    const float *__restrict__ qkv, const int32_t *__restrict__ pos0, int heads,
+    const __half *__restrict__ kcache, const __half *__restrict__ vcache, int max_seq,
+    float *__restrict__ out) {
+    constexpr int hd = 128;
+    __shared__ float s_q[hd];
+    __shared__ float s_p[kWaves][64];
+    __shared__ float s_m[kWaves], s_l[kWaves];
+    __shared__ float s_o[kWaves][hd];
+    const int m = blockIdx.x / heads, h = blockIdx.x - m * heads;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int HD = heads * hd;
+    int p = pos0[0] + m;
+    if (p >= max_seq) p = max_seq - 1;
+    const int nkeys = p + 1;
+    const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
+    if (tid < hd) s_q[tid] = qkv[(size_t)m * 3 * HD + h * hd + tid] * scale;
+    __syncthreads();
+
+    const __half *kh = kcache + (size_t)h * max_seq * hd;
+    const __half *vh = vcache + (size_t)h * max_seq * hd;
+    float run_max = -INFINITY, run_sum = 0.0f, o0 = 0.0f, o1 = 0.0f;
+    for (int t0 = wave * 64; t0 < nkeys; t0 += kWaves * 64) {
+        const int t = t0 + lane;
+        float s = -INFINITY;
+        if (t < nkeys) {
+            const uint4 *krow = reinterpret_cast<const uint4 *>(kh + (size_t)t * hd);
+            float acc = 0.0f;
+#pragma unroll
+            for (int c = 0; c < hd / 8; ++c) {
+                const uint4 u = krow[c];
+                const __half2 *h2 = reinterpret_cast<const __half2 *>(&u);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float2 f = __half22float2(h2[e]);
+                    acc = fmaf(f.x, s_q[c * 8 + 2 * e], acc);
+                    acc = fmaf(f.y, s_q[c * 8 + 2 * e + 1], acc);
+                }
+            }
+            s = acc;
+        }
+        const float blk_max = wave_max_f(s);
+        const float new_max = fmaxf(run_max, blk_max);
+        const float corr = __expf(run_max - new_max);  // 0 on the first block
+        const float pr = t < nkeys ? __expf(s - new_max) : 0.0f;
+        run_sum = run_sum * corr + wave_sum_f(pr);
+        run_max = new_max;
+        o0 *= corr;
+        o1 *= corr;
+        s_p[wave][lane] = pr;
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const int cnt = min(64, nkeys - t0);
+        for (int j = 0; j < cnt; ++j) {
+            const float pj = s_p[wave][j];
+            const float2 v = __half22float2(
+                *reinterpret_cast<const __half2 *>(vh + (size_t)(t0 + j) * hd + 2 * lane));
+            o0 = fmaf(pj, v.x, o0);
+            o1 = fmaf(pj, v.y, o1);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (lane == 0) {
+        s_m[wave] = run_max;
+        s_l[wave] = run_sum;
+    }
+    s_o[wave][2 * lane] = o0;
+    s_o[wave][2 * lane + 1] = o1;
+    __syncthreads();
+    if (tid < hd) {
+        float gmax = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) gmax = fmaxf(gmax, s_m[w]);
+        float num = 0.0f, den = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+            const float c = s_m[w] == -INFINITY ? 0.0f : __expf(s_m[w] - gmax);
+            num += c * s_o[w][tid];
+            den += c * s_l[w];
+        }
+        out[(size_t)m * HD + h * hd + tid] = num / den;
+    }
+}
+
+// h[m, f] = silu(gu[m, f]) * gu[m, F + f]
+__global__ __launch_bounds__(kBlock) void swiglu_kernel(const float *__restrict__ gu, int F,
+                                                        float *__restrict__ hout) {
+    const int m = blockIdx.y;
+    const int f = blockIdx.x * kBlock + threadIdx.x;
+    if (f < F) {
+        const float g = gu[(size_t)m * 2 * F + f], u = gu[(size_t)m * 2 * F + F + f];
+        hout[(size_t)m * F + f] = (g / (1.0f + __expf(-g))) * u;
+    }
+}
+
+// Index of the largest of n values (the lowest index among equals); one workgroup.
+__global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ v, int n,
+                                                      int32_t *__restrict__ out,
+                                                      int32_t *__restrict__ hist,
+                                                      const int32_t *__restrict__ hist_pos) {
+    __shared__ float s_v[16];
+    __shared__ int s_i[16];
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += 1024) {
+        const float x = v[i];
+        if (x > best || (x == best && i < bi)) {
+            best = x;
+            bi = i;
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ob = __shfl_xor(best, off);
+        const int oi = __shfl_xor(bi, off);
+        if (ob > best || (ob == best && oi < bi)) {
+            best = ob;
+            bi = oi;
+        }
+    }
+    if ((threadIdx.x & 63) == 0) {
+        s_v[threadIdx.x >> 6] = best;
+        s_i[threadIdx.x >> 6] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; ++w)
+            if (s_v[w] > best || (s_v[w] == best && s_i[w] < bi)) {
+                best = s_v[w];
+                bi = s_i[w];
+            }
+        bi = bi == 0x7fffffff ? 0 : bi;
+        out[0] = bi;
+        if (hist) hist[hist_pos[0]] = bi;
+    }
+}
+
+__global__ void add_i32_kernel(int32_t *p, int delta) { p[0] += delta; }
+
+// out[i] = sigma * z_i, z_i standard normal from a counter-based generator (splitmix64 of
+// (seed, i / 2), Box-Muller in f32).  For random-initialised weights that never leave the
+// device; NOT the host generator of rbn_synth_normal_f32.
+__global__ __launch_bounds__(kBlock) void synth_normal_device_kernel(uint64_t seed, float sigma,
+                                                                     float *__restrict__ out,
+                                                                     uint64_t n) {
+    const uint64_t pair = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (2 * pair >= n) return;
+    uint64_t z = seed * 0x9E3779B97F4A7C15ull + (pair + 1) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    const float u1 = ((float)(uint32_t)(z >> 40) + 1.0f) * (1.0f / 16777216.0f);  // (0, 1]
+    const float u2 = (float)(uint32_t)((z >> 16) & 0xFFFFFF) * (1.0f / 16777216.0f);
+    const float r = sqrtf(-2.0f * __logf(u1)) * sigma;
+    float sn, cs;
+    sincosf(6.283185307179586f * u2, &sn, &cs);
+    out[2 * pair] = r * cs;
+    if (2 * pair + 1 < n) out[2 * pair + 1] = r * sn;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rbn_embed_f32(rbn_ctx *ctx, const float *d_table, const int32_t *d_tokens, uint64_t M,
+                  uint64_t H, uint64_t vocab, float *d_x) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(d_table && d_tokens && d_x, "null pointer in rbn_embed_f32");
+    RBN_REQUIRE(M > 0 && M < (1u << 20) && H > 0 && H < (1u << 24) && vocab > 0 && vocab < (1u << 30),
+                "bad sizes in rbn_embed_f32");
+    embed_kernel<<<dim3((unsigned)M), dim3(kBlock), 0, ctx->stream>>>(d_table, d_tokens, (int)H,
+                                                                     (int)vocab, d_x);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+int rbn_rmsnorm_quant_i8(rbn_ctx *ctx, float *d_x, const float *d_delta, const float *d_gamma,
+                         float eps, uint64_t M, uint64_t H, int8_t *d_q, float *d_act_scale,
+                         int32_t *d_rowsum) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(d_x && d_gamma && d_q && d_act_scale && d_rowsum, "null pointer in rbn_rmsnorm_quant_i8");
+    RBN_REQUIRE(M > 0 && M < (1u << 20), "bad M in rbn_rmsnorm_quant_i8");
+    const uint64_t pitch = rbn_kpad(H);
+    RBN_REQUIRE(H > 0 && pitch <= (uint64_t)kBlock * kPer, "rbn_rmsnorm_quant_i8 takes H <= %d",
+                kBlock * kPer);
+    rmsnorm_quant_kernel<<<dim3((unsigned)M), dim3(kBlock), 0, ctx->stream>>>(
+        d_x, d_delta, d_gamma, eps, (int)H, (int)pitch, d_q, d_act_scale, d_rowsum);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+int rbn_rope_kv_store_f16(rbn_ctx *ctx, float *d_qkv, const int32_t *d_pos0, uint64_t M,
+                          uint64_t heads, uint64_t head_dim, float theta, void *d_kcache,
+                          void *d_vcache, uint64_t max_seq) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(d_qkv && d_pos0 && d_kcache && d_vcache, "null pointer in rbn_rope_kv_store_f16");
+    RBN_REQUIRE(M > 0 && M < (1u << 20) && heads > 0 && heads < 4096 && head_dim >= 2 &&
+                    head_dim <= 1024 && (head_dim & 1) == 0 && max_seq > 0 && max_seq < (1u << 24),
+                "bad sizes in rbn_rope_kv_store_f16");
+    rope_kv_store_kernel<<<dim3((unsigned)M), dim3(kBlock), 0, ctx->stream>>>(
+        d_qkv, d_pos0, (int)heads, (int)head_dim, theta, (__half *)d_kcache, (__half *)d_vcache,
+        (int)max_seq);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+int rbn_attention_f16kv(rbn_ctx *ctx, const float *d_qkv, const int32_t *d_pos0, uint64_t M,
+                        uint64_t heads, uint64_t head_dim, const void *d_kcache,
+                        const void *d_vcache, uint64_t max_seq, float *d_out) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(d_qkv && d_pos0 && d_kcache && d_vcache && d_out, "null pointer in rbn_attention_f16kv");
+    RBN_REQUIRE(head_dim == 128, "rbn_attention_f16kv takes head_dim == 128 (got %llu)",
+                (unsigned long long)head_dim);
+    RBN_REQUIRE(M > 0 && heads > 0 && M * heads < (1ull << 31) && max_seq > 0 && max_seq < (1u << 24),
+                "bad sizes in rbn_attention_f16kv");
+    // a single token (decode) gets more waves per head: only `heads` workgroups run
+    if (M == 1)
+        attention_kernel<16><<<dim3((unsigned)(M * heads)), dim3(16 * 64), 0, ctx->stream>>>(
+            d_qkv, d_pos0, (int)heads, (const __half *)d_kcache, (const __half *)d_vcache, (int)max_seq, d_out);
+    else
+        attention_kernel<4><<<dim3((unsigned)(M * heads)), dim3(4 * 64), 0, ctx->stream>>>(
+            d_qkv, d_pos0, (int)heads, (const __half *)d_kcache, (const __half *)d_vcache, (int)max_seq, d_out);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+int rbn_swiglu_f32(rbn_ctx *ctx, const float *d_gate_up, uint64_t M, uint64_t F, float *d_h) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(d_gate_up && d_h, "null pointer in rbn_swiglu_f32");
+    RBN_REQUIRE(M > 0 && M < 65536 && F > 0 && F < (1u << 24), "bad sizes in rbn_swiglu_f32");
+    swiglu_kernel<<<dim3((unsigned)((F + kBlock - 1) / kBlock), (unsigned)M), dim3(kBlock), 0, ctx->stream>>>(
+        d_gate_up, (int)F, d_h);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+int rbn_argmax_f32(rbn_ctx *ctx, const float *d_values, uint64_t n, int32_t *d_index,
+                   int32_t *d_history, const int32_t *d_history_pos) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(d_values && d_index, "null pointer in rbn_argmax_f32");
+    RBN_REQUIRE(n > 0 && n < (1u << 30), "bad n in rbn_argmax_f32");
+    RBN_REQUIRE((d_history == nullptr) == (d_history_pos == nullptr),
+                "d_history and d_history_pos go together");
+    argmax_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(d_values, (int)n, d_index, d_history,
+                                                          d_history_pos);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+int rbn_add_i32(rbn_ctx *ctx, int32_t *d_value, int32_t delta) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(d_value != nullptr, "null pointer in rbn_add_i32");
+    add_i32_kernel<<<dim3(1), dim3(1), 0, ctx->stream>>>(d_value, delta);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+int rbn_synth_normal_device_f32(rbn_ctx *ctx, uint64_t seed, float sigma, float *d_out, uint64_t n) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(d_out != nullptr && n > 0, "bad arguments in rbn_synth_normal_device_f32");
+    const uint64_t pairs = (n + 1) / 2, blocks = (pairs + kBlock - 1) / kBlock;
+    RBN_REQUIRE(blocks < (1ull << 31), "n too large");
+    synth_normal_device_kernel<<<dim3((unsigned)blocks), dim3(kBlock), 0, ctx->stream>>>(seed, sigma, d_out, n);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+}  // extern "C"

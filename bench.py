@@ -151,6 +151,44 @@ def time_ternarize(ctx, K, N, sigma):
     return out
 
 
+def time_decoder(ctx, prompt_len=512, new_tokens=128, use_graph=True):
+    """BitNet-b1.58 2B-class decoder, random-initialised on the device: 24 layers, hidden
+    2560, 20 heads of 128, SwiGLU FFN 6912, vocabulary 32000, f16 K/V.  Batch 1: a prompt of
+    prompt_len tokens, then new_tokens greedy tokens replayed from one captured HIP graph."""
+    from ronn_amd.decoder import BitNetDecoder, DecoderConfig
+    cfg = DecoderConfig(max_seq=prompt_len + new_tokens + 8)
+    dec = BitNetDecoder(ctx, cfg, max_batch_tokens=prompt_len)
+    t0 = time.perf_counter()
+    dec.init_random(seed=4)
+    t_init = time.perf_counter() - t0
+    prompt = (np.arange(prompt_len, dtype=np.int64) * 7919 % cfg.vocab).astype(np.int32)
+    dec.prefill(prompt)       # warm-up (also sizes every workspace before the capture)
+    ctx.sync()
+    t0 = time.perf_counter()
+    dec.prefill(prompt)
+    ctx.sync()
+    t_prefill = time.perf_counter() - t0
+    dec.decode(4, use_graph)  # captures the graph, warms it up
+    dec.prefill(prompt)
+    tokens, dt = dec.decode(new_tokens, use_graph)
+    w_bytes = cfg.packed_weight_bytes_per_token()
+    kv_bytes = 2 * 2 * cfg.layers * cfg.attn_dim * (prompt_len + new_tokens / 2.0)   # average over the run
+    per_tok = dt / new_tokens
+    return {"config": dataclass_dict(cfg), "prompt_tokens": prompt_len, "new_tokens": new_tokens,
+            "decode_tok_per_s": new_tokens / dt, "ms_per_token": per_tok * 1e3,
+            "prefill_ms": t_prefill * 1e3, "prefill_tok_per_s": prompt_len / t_prefill,
+            "weight_init_s": t_init, "launches_per_token": 9 * cfg.layers + 5,
+            "bytes_per_token": {"packed_weights": w_bytes, "kv_cache_f16_avg": kv_bytes},
+            "GBps": (w_bytes + kv_bytes) / per_tok / 1e9,
+            "frac_hbm_peak": (w_bytes + kv_bytes) / per_tok / 1e9 / HBM_PEAK_GBS,
+            "first_tokens": [int(t) for t in tokens[:8]]}
+
+
+def dataclass_dict(obj):
+    import dataclasses
+    return dataclasses.asdict(obj)
+
+
 def cpu_baseline(wl, out, acc, budget_s=20.0):
     """Times the CPU oracle on the headline inputs (one core) and gates parity."""
     from oracle import oracle as O
@@ -221,6 +259,11 @@ def profile_kernel(ctx, which, launches):
                 ctx.pack_ternary(d_w, K * N, 0.0028, d_p)
             else:
                 ctx.quantize_ternary(d_w, K * N, _lib.SUM_STRICT_SEQ, d_p)
+    elif which in ("decoder", "decoder_eager"):
+        # decoder_eager launches kernel by kernel instead of replaying the captured graph
+        # (for per-kernel traces: the profiler does not survive the 269-node graph)
+        print(json.dumps(time_decoder(ctx, new_tokens=min(launches, 32), use_graph=which == "decoder")))
+        return
     elif which == "copy":
         n = 256 << 20
         a, b = ctx.alloc(n), ctx.alloc(n)
@@ -238,7 +281,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=400)
     ap.add_argument("--no-extra", action="store_true", help="headline only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline / parity gate")
-    ap.add_argument("--kernel", choices=["gemv", "skinny", "gemm", "pack", "quantize", "copy"],
+    ap.add_argument("--kernel", choices=["gemv", "skinny", "gemm", "pack", "quantize", "copy", "decoder", "decoder_eager"],
                     help="profiling aid: launch only this kernel a few times (for rocprofv3) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -336,6 +379,7 @@ def main():
         extra["mfma_i8_probe_TOPS"] = {"constant_operands": ctx.probe_mfma_i8(0),
                                        "int8_x_ternary_codes": ctx.probe_mfma_i8(1),
                                        "int8_x_int8": ctx.probe_mfma_i8(2)}
+        extra["decoder"] = time_decoder(ctx)
         result["extra"] = extra
 
     print(json.dumps(result))

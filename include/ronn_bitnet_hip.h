@@ -222,12 +222,14 @@ int rbn_execute_ternary_matmul(rbn_ctx *ctx, const float *h_a, const float *h_b,
 /* x[m,:] = table[tokens[m],:] (token ids clamped to [0, vocab)). */
 int rbn_embed_f32(rbn_ctx *ctx, const float *d_table, const int32_t *d_tokens, uint64_t M,
                   uint64_t H, uint64_t vocab, float *d_x);
-/* If d_delta: x += delta, written back (residual stream).  Then
+/* Input row: x[m,:] (H values); or, when d_delta is given, x += delta, written back
+ * (the residual stream); or, when d_gate_up [M, 2H] is given instead of d_x,
+ * x = silu(gate) * up (SwiGLU on the way in; nothing is written back).  Then
  * y = (x * rsqrt(mean(x^2) + eps)) * gamma, quantised per token exactly as
  * rbn_act_quant_i8 does (same output format).  H <= 8192. */
-int rbn_rmsnorm_quant_i8(rbn_ctx *ctx, float *d_x, const float *d_delta, const float *d_gamma,
-                         float eps, uint64_t M, uint64_t H, int8_t *d_q, float *d_act_scale,
-                         int32_t *d_rowsum);
+int rbn_rmsnorm_quant_i8(rbn_ctx *ctx, float *d_x, const float *d_delta, const float *d_gate_up,
+                         const float *d_gamma, float eps, uint64_t M, uint64_t H, int8_t *d_q,
+                         float *d_act_scale, int32_t *d_rowsum);
 /* d_qkv [M, 3*heads*head_dim] = (q | k | v).  Rotary embedding (pairs
  * (i, i + head_dim/2), angle pos * theta^(-2i/head_dim), pos = *d_pos0 + m) of q in
  * place and of k on its way into the cache: rotated k and v go to the f16 caches
@@ -240,6 +242,11 @@ int rbn_rope_kv_store_f16(rbn_ctx *ctx, float *d_qkv, const int32_t *d_pos0, uin
 int rbn_attention_f16kv(rbn_ctx *ctx, const float *d_qkv, const int32_t *d_pos0, uint64_t M,
                         uint64_t heads, uint64_t head_dim, const void *d_kcache,
                         const void *d_vcache, uint64_t max_seq, float *d_out);
+/* One token: rbn_rope_kv_store_f16 and rbn_attention_f16kv in one launch (d_qkv is
+ * not modified: the rotated q stays inside the kernel). */
+int rbn_attention_decode_f16kv(rbn_ctx *ctx, const float *d_qkv, const int32_t *d_pos, uint64_t heads,
+                               uint64_t head_dim, float theta, void *d_kcache, void *d_vcache,
+                               uint64_t max_seq, float *d_out);
 /* h[m,f] = silu(gu[m,f]) * gu[m,F+f], gu [M, 2F]. */
 int rbn_swiglu_f32(rbn_ctx *ctx, const float *d_gate_up, uint64_t M, uint64_t F, float *d_h);
 /* *d_index = index of the largest value (lowest index among equals).  If d_history

@@ -91,9 +91,10 @@ SIGNATURES = {
     "rbn_gemm_t2_i8_skinny": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
     "rbn_gemm_t2_i8_mfma": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
     "rbn_embed_f32": (C.c_int, [_vp, _vp, _vp, _u64, _u64, _u64, _vp]),
-    "rbn_rmsnorm_quant_i8": (C.c_int, [_vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _vp, _vp, _vp]),
+    "rbn_rmsnorm_quant_i8": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _vp, _vp, _vp]),
     "rbn_rope_kv_store_f16": (C.c_int, [_vp, _vp, _vp, _u64, _u64, _u64, C.c_float, _vp, _vp, _u64]),
     "rbn_attention_f16kv": (C.c_int, [_vp, _vp, _vp, _u64, _u64, _u64, _vp, _vp, _u64, _vp]),
+    "rbn_attention_decode_f16kv": (C.c_int, [_vp, _vp, _vp, _u64, _u64, C.c_float, _vp, _vp, _u64, _vp]),
     "rbn_swiglu_f32": (C.c_int, [_vp, _vp, _u64, _u64, _vp]),
     "rbn_argmax_f32": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _vp]),
     "rbn_add_i32": (C.c_int, [_vp, _vp, C.c_int32]),

@@ -39,76 +39,98 @@ __global__ __launch_bounds__(kBlock) void embed_kernel(const float *__restrict__
     for (int i = threadIdx.x; i < H; i += kBlock) x[(size_t)m * H + i] = src[i];
 }
 
-// One workgroup per token:
-//   if delta: x += delta (written back: the residual stream)
-//   y = x * rsqrt(mean(x^2) + eps) * gamma
+// One workgroup of 1024 threads per token:
+//   x = silu(gate) * up   when gate_up is given (SwiGLU computed on the way in), else
+//   x += delta            when delta is given (written back: the residual stream)
+//   y = (x * rsqrt(mean(x^2) + eps)) * gamma
 //   g = max(max|y|, 1e-5); q = clamp(rne(y * (127/g)), -128, 127); scale = g/127; rowsum = sum q
-// The row (H <= kBlock * kPer floats) stays in registers between the passes.
-constexpr int kPer = 32;  // H <= 8192
-__global__ __launch_bounds__(kBlock) void rmsnorm_quant_kernel(
-    float *__restrict__ x, const float *__restrict__ delta, const float *__restrict__ gamma,
-    float eps, int H, int pitch, int8_t *__restrict__ q, float *__restrict__ act_scale,
-    int32_t *__restrict__ rowsum) {
-    __shared__ float s_red[kBlock / 64];
-    __shared__ int s_redi[kBlock / 64];
+// With one token the kernel is a chain of memory round trips, so every load (row, delta,
+// gains) is issued before the first reduction and the row stays in registers.
+constexpr int kNormThreads = 1024;
+constexpr int kPer = 8;  // H <= 8192
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_quant_kernel(
+    float *__restrict__ x, const float *__restrict__ delta, const float *__restrict__ gate_up,
+    const float *__restrict__ gamma, float eps, int H, int pitch, int8_t *__restrict__ q,
+    float *__restrict__ act_scale, int32_t *__restrict__ rowsum) {
+    __shared__ float s_red[kNormThreads / 64];
+    __shared__ int s_redi[kNormThreads / 64];
     const int m = blockIdx.x, tid = threadIdx.x;
-    float *row = x + (size_t)m * H;
-    const float *drow = delta ? delta + (size_t)m * H : nullptr;
-    float v[kPer];
-    float ss = 0.0f;
+    float v[kPer], gm[kPer];
+    if (gate_up) {
+        const float *gu = gate_up + (size_t)m * 2 * H;
 #pragma unroll
-    for (int j = 0; j < kPer; ++j) {
-        const int i = tid + j * kBlock;
-        float t = 0.0f;
-        if (i < H) {
-            t = row[i];
-            if (drow) {
-                t += drow[i];
-                row[i] = t;
+        for (int j = 0; j < kPer; ++j) {
+            const int i = tid + j * kNormThreads;
+            const float g = i < H ? gu[i] : 0.0f, u = i < H ? gu[H + i] : 0.0f;
+            gm[j] = i < H ? gamma[i] : 0.0f;
+            v[j] = (g / (1.0f + __expf(-g))) * u;
+        }
+    } else {
+        float *row = x + (size_t)m * H;
+        const float *drow = delta ? delta + (size_t)m * H : nullptr;
+        float dv[kPer];
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+            const int i = tid + j * kNormThreads;
+            v[j] = i < H ? row[i] : 0.0f;
+            dv[j] = (drow && i < H) ? drow[i] : 0.0f;
+            gm[j] = i < H ? gamma[i] : 0.0f;
+        }
+        if (drow) {
+#pragma unroll
+            for (int j = 0; j < kPer; ++j) {
+                const int i = tid + j * kNormThreads;
+                v[j] += dv[j];
+                if (i < H) row[i] = v[j];
             }
         }
-        v[j] = t;
-        ss += t * t;
     }
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) ss += v[j] * v[j];
     ss = wave_sum_f(ss);
     if ((tid & 63) == 0) s_red[tid >> 6] = ss;
     __syncthreads();
-    ss = (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
+    ss = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kNormThreads / 64; ++w) ss += s_red[w];
     const float inv_rms = 1.0f / sqrtf(ss / (float)H + eps);
     float amax = 0.0f;
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
-        const int i = tid + j * kBlock;
-        const float y = i < H ? (v[j] * inv_rms) * gamma[i] : 0.0f;
-        v[j] = y;
-        amax = fmaxf(amax, fabsf(y));
+        v[j] = (v[j] * inv_rms) * gm[j];
+        amax = fmaxf(amax, fabsf(v[j]));
     }
     amax = wave_max_f(amax);
     __syncthreads();
     if ((tid & 63) == 0) s_red[tid >> 6] = amax;
     __syncthreads();
-    amax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    amax = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kNormThreads / 64; ++w) amax = fmaxf(amax, s_red[w]);
     const float gmax = fmaxf(amax, 1e-5f);
     const float inv = 127.0f / gmax;
     int sum = 0;
     int8_t *qrow = q + (size_t)m * pitch;
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
-        const int i = tid + j * kBlock;
+        const int i = tid + j * kNormThreads;
         if (i < pitch) {
-            float r = rintf(v[j] * inv);  // round half to even; 0 in the padding
+            float r = rintf(v[j] * inv);  // round half to even; v is 0 in the padding
             r = fminf(fmaxf(r, -128.0f), 127.0f);
-            const int qi = i < H ? (int)r : 0;
-            qrow[i] = (int8_t)qi;
-            sum += qi;
+            qrow[i] = (int8_t)(int)r;
+            sum += (int)r;
         }
     }
     sum = wave_sum_i(sum);
     if ((tid & 63) == 0) s_redi[tid >> 6] = sum;
     __syncthreads();
     if (tid == 0) {
+        int tot = 0;
+#pragma unroll
+        for (int w = 0; w < kNormThreads / 64; ++w) tot += s_redi[w];
         act_scale[m] = gmax / 127.0f;
-        rowsum[m] = (s_redi[0] + s_redi[1]) + (s_redi[2] + s_redi[3]);
+        rowsum[m] = tot;
     }
 }
 
@@ -149,10 +171,12 @@ __global__ __launch_bounds__(kBlock) void rope_kv_store_kernel(
 // One workgroup per (m, h); hd == 128.  Each wave takes every kWaves-th block of 64 keys:
 // scores with one key per lane (the key row is read as 16 x 16 bytes), online softmax,
 // then P.V with two dimensions per lane; the waves' (max, sum, out) meet through LDS.
-template <int kWaves>
+// FUSED (single token): the workgroup first rotates its head's q and k, writes k and v to
+// the cache (what rope_kv_store_kernel does) and then attends, one launch instead of two.
+template <int kWaves, bool FUSED>
 __global__ __launch_bounds__(kWaves * 64) void attention_kernel(
-    const float *__restrict__ qkv, const int32_t *__restrict__ pos0, int heads,
-    const __half *__restrict__ kcache, const __half *__restrict__ vcache, int max_seq,
+    const float *__restrict__ qkv, const int32_t *__restrict__ pos0, int heads, float theta,
+    __half *__restrict__ kcache, __half *__restrict__ vcache, int max_seq,
     float *__restrict__ out) {
     constexpr int hd = 128;
     __shared__ float s_q[hd];
@@ -166,8 +190,26 @@ __global__ __launch_bounds__(kWaves * 64) void attention_kernel(
     if (p >= max_seq) p = max_seq - 1;
     const int nkeys = p + 1;
     const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
-    if (tid < hd) s_q[tid] = qkv[(size_t)m * 3 * HD + h * hd + tid] * scale;
-    __syncthreads();
+    if (FUSED) {
+        if (tid < hd / 2) {
+            const int i = tid, half = hd / 2;
+            const float freq = powf(theta, -2.0f * (float)i / (float)hd);
+            float sn, cs;
+            sincosf((float)p * freq, &sn, &cs);
+            const float *qh = qkv + (size_t)m * 3 * HD + h * hd, *kh_new = qh + HD, *vh_new = qh + 2 * HD;
+            const float q0 = qh[i], q1 = qh[i + half], k0 = kh_new[i], k1 = kh_new[i + half];
+            s_q[i] = (q0 * cs - q1 * sn) * scale;
+            s_q[i + half] = (q1 * cs + q0 * sn) * scale;
+            const size_t c = ((size_t)h * max_seq + p) * hd;
+            kcache[c + i] = __float2half_rn(k0 * cs - k1 * sn);
+            kcache[c + i + half] = __float2half_rn(k1 * cs + k0 * sn);
+            vcache[c + i] = __float2half_rn(vh_new[i]);
+            vcache[c + i + half] = __float2half_rn(vh_new[i + half]);
+        }
+    } else {
+        if (tid < hd) s_q[tid] = qkv[(size_t)m * 3 * HD + h * hd + tid] * scale;
+    }
+    __syncthreads();  // also makes the new cache row visible to the whole workgroup
 
     const __half *kh = kcache + (size_t)h * max_seq * hd;
     const __half *vh = vcache + (size_t)h * max_seq * hd;
@@ -202,13 +244,21 @@ __global__ __launch_bounds__(kWaves * 64) void attention_kernel(
         s_p[wave][lane] = pr;
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        const int cnt = min(64, nkeys - t0);
-        for (int j = 0; j < cnt; ++j) {
-            const float pj = s_p[wave][j];
-            const float2 v = __half22float2(
-                *reinterpret_cast<const __half2 *>(vh + (size_t)(t0 + j) * hd + 2 * lane));
-            o0 = fmaf(pj, v.x, o0);
-            o1 = fmaf(pj, v.y, o1);
+        // eight value rows per round, loads first; rows past the end repeat the last one
+        // with probability 0
+        const int last = nkeys - 1 - t0;
+        for (int j0 = 0; j0 <= min(63, last); j0 += 8) {
+            __half2 vr[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                vr[u] = *reinterpret_cast<const __half2 *>(vh + (size_t)(t0 + min(j0 + u, last)) * hd + 2 * lane);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const float pj = s_p[wave][j0 + u];  // 0 beyond the last key
+                const float2 v = __half22float2(vr[u]);
+                o0 = fmaf(pj, v.x, o0);
+                o1 = fmaf(pj, v.y, o1);
+            }
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -326,17 +376,20 @@ int rbn_embed_f32(rbn_ctx *ctx, const float *d_table, const int32_t *d_tokens, u
     return RBN_OK;
 }
 
-int rbn_rmsnorm_quant_i8(rbn_ctx *ctx, float *d_x, const float *d_delta, const float *d_gamma,
-                         float eps, uint64_t M, uint64_t H, int8_t *d_q, float *d_act_scale,
-                         int32_t *d_rowsum) {
+int rbn_rmsnorm_quant_i8(rbn_ctx *ctx, float *d_x, const float *d_delta, const float *d_gate_up,
+                         const float *d_gamma, float eps, uint64_t M, uint64_t H, int8_t *d_q,
+                         float *d_act_scale, int32_t *d_rowsum) {
     RBN_ENTER(ctx);
-    RBN_REQUIRE(d_x && d_gamma && d_q && d_act_scale && d_rowsum, "null pointer in rbn_rmsnorm_quant_i8");
+    RBN_REQUIRE(d_gamma && d_q && d_act_scale && d_rowsum, "null pointer in rbn_rmsnorm_quant_i8");
+    RBN_REQUIRE((d_x != nullptr) != (d_gate_up != nullptr),
+                "rbn_rmsnorm_quant_i8 takes either d_x (with optional d_delta) or d_gate_up");
+    RBN_REQUIRE(d_gate_up == nullptr || d_delta == nullptr, "d_delta goes with d_x only");
     RBN_REQUIRE(M > 0 && M < (1u << 20), "bad M in rbn_rmsnorm_quant_i8");
     const uint64_t pitch = rbn_kpad(H);
-    RBN_REQUIRE(H > 0 && pitch <= (uint64_t)kBlock * kPer, "rbn_rmsnorm_quant_i8 takes H <= %d",
-                kBlock * kPer);
-    rmsnorm_quant_kernel<<<dim3((unsigned)M), dim3(kBlock), 0, ctx->stream>>>(
-        d_x, d_delta, d_gamma, eps, (int)H, (int)pitch, d_q, d_act_scale, d_rowsum);
+    RBN_REQUIRE(H > 0 && pitch <= (uint64_t)kNormThreads * kPer, "rbn_rmsnorm_quant_i8 takes H <= %d",
+                kNormThreads * kPer);
+    rmsnorm_quant_kernel<<<dim3((unsigned)M), dim3(kNormThreads), 0, ctx->stream>>>(
+        d_x, d_delta, d_gate_up, d_gamma, eps, (int)H, (int)pitch, d_q, d_act_scale, d_rowsum);
     RBN_HIP(hipGetLastError());
     return RBN_OK;
 }
@@ -367,11 +420,26 @@ int rbn_attention_f16kv(rbn_ctx *ctx, const float *d_qkv, const int32_t *d_pos0,
                 "bad sizes in rbn_attention_f16kv");
     // a single token (decode) gets more waves per head: only `heads` workgroups run
     if (M == 1)
-        attention_kernel<16><<<dim3((unsigned)(M * heads)), dim3(16 * 64), 0, ctx->stream>>>(
-            d_qkv, d_pos0, (int)heads, (const __half *)d_kcache, (const __half *)d_vcache, (int)max_seq, d_out);
+        attention_kernel<16, false><<<dim3((unsigned)(M * heads)), dim3(16 * 64), 0, ctx->stream>>>(
+            d_qkv, d_pos0, (int)heads, 0.0f, (__half *)d_kcache, (__half *)d_vcache, (int)max_seq, d_out);
     else
-        attention_kernel<4><<<dim3((unsigned)(M * heads)), dim3(4 * 64), 0, ctx->stream>>>(
-            d_qkv, d_pos0, (int)heads, (const __half *)d_kcache, (const __half *)d_vcache, (int)max_seq, d_out);
+        attention_kernel<4, false><<<dim3((unsigned)(M * heads)), dim3(4 * 64), 0, ctx->stream>>>(
+            d_qkv, d_pos0, (int)heads, 0.0f, (__half *)d_kcache, (__half *)d_vcache, (int)max_seq, d_out);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+int rbn_attention_decode_f16kv(rbn_ctx *ctx, const float *d_qkv, const int32_t *d_pos, uint64_t heads,
+                               uint64_t head_dim, float theta, void *d_kcache, void *d_vcache,
+                               uint64_t max_seq, float *d_out) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(d_qkv && d_pos && d_kcache && d_vcache && d_out, "null pointer in rbn_attention_decode_f16kv");
+    RBN_REQUIRE(head_dim == 128, "rbn_attention_decode_f16kv takes head_dim == 128 (got %llu)",
+                (unsigned long long)head_dim);
+    RBN_REQUIRE(heads > 0 && heads < 4096 && max_seq > 0 && max_seq < (1u << 24),
+                "bad sizes in rbn_attention_decode_f16kv");
+    attention_kernel<16, true><<<dim3((unsigned)heads), dim3(16 * 64), 0, ctx->stream>>>(
+        d_qkv, d_pos, (int)heads, theta, (__half *)d_kcache, (__half *)d_vcache, (int)max_seq, d_out);
     RBN_HIP(hipGetLastError());
     return RBN_OK;
 }

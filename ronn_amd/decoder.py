@@ -69,7 +69,6 @@ class BitNetDecoder:
         self.qkv = a(4 * T * 3 * A)
         self.att = a(4 * T * A)
         self.gu = a(4 * T * 2 * F)
-        self.h = a(4 * T * F)
         self.logits = a(4 * V)
         pitch = ctx.act_pitch(max(H, A, F))
         self.acts = (a(T * pitch), a(4 * T), a(4 * T))
@@ -153,10 +152,12 @@ class BitNetDecoder:
         ctx.sync()
 
     # -- one forward pass over M tokens starting at the position in self.pos -----------------
-    def _norm_quant(self, x: DeviceBuffer, delta, gamma: DeviceBuffer, M: int, H: int, row0: int = 0):
+    def _norm_quant(self, x, delta, gamma: DeviceBuffer, M: int, H: int, row0: int = 0, gate_up=None):
         off = 4 * row0 * H
         check(self.lib.rbn_rmsnorm_quant_i8(
-            self.ctx.handle, x.ptr + off, (delta.ptr + off) if delta is not None else None, gamma.ptr,
+            self.ctx.handle, (x.ptr + off) if x is not None else None,
+            (delta.ptr + off) if delta is not None else None,
+            gate_up.ptr if gate_up is not None else None, gamma.ptr,
             self.cfg.eps, M, H, self.acts[0].ptr, self.acts[1].ptr, self.acts[2].ptr))
 
     def _linear(self, lin: _Linear, M: int, out: DeviceBuffer):
@@ -174,18 +175,22 @@ class BitNetDecoder:
         for i, b in enumerate(self.blocks):
             self._norm_quant(self.x, pending, b["g_attn"], M, H)
             self._linear(b["wqkv"], M, self.qkv)
-            check(lib.rbn_rope_kv_store_f16(hnd, self.qkv.ptr, self.pos.ptr, M, cfg.heads, cfg.head_dim,
-                                            cfg.rope_theta, self.kcache[i].ptr, self.vcache[i].ptr,
-                                            cfg.max_seq))
-            check(lib.rbn_attention_f16kv(hnd, self.qkv.ptr, self.pos.ptr, M, cfg.heads, cfg.head_dim,
-                                          self.kcache[i].ptr, self.vcache[i].ptr, cfg.max_seq,
-                                          self.att.ptr))
+            if M == 1:
+                check(lib.rbn_attention_decode_f16kv(hnd, self.qkv.ptr, self.pos.ptr, cfg.heads, cfg.head_dim,
+                                                     cfg.rope_theta, self.kcache[i].ptr, self.vcache[i].ptr,
+                                                     cfg.max_seq, self.att.ptr))
+            else:
+                check(lib.rbn_rope_kv_store_f16(hnd, self.qkv.ptr, self.pos.ptr, M, cfg.heads, cfg.head_dim,
+                                                cfg.rope_theta, self.kcache[i].ptr, self.vcache[i].ptr,
+                                                cfg.max_seq))
+                check(lib.rbn_attention_f16kv(hnd, self.qkv.ptr, self.pos.ptr, M, cfg.heads, cfg.head_dim,
+                                              self.kcache[i].ptr, self.vcache[i].ptr, cfg.max_seq,
+                                              self.att.ptr))
             self._norm_quant(self.att, None, b["g_attn_sub"], M, A)
             self._linear(b["wo"], M, self.o)
             self._norm_quant(self.x, self.o, b["g_ffn"], M, H)
             self._linear(b["wgu"], M, self.gu)
-            check(lib.rbn_swiglu_f32(hnd, self.gu.ptr, M, F, self.h.ptr))
-            self._norm_quant(self.h, None, b["g_ffn_sub"], M, F)
+            self._norm_quant(None, None, b["g_ffn_sub"], M, F, gate_up=self.gu)   # SwiGLU fused in
             self._linear(b["wdown"], M, self.d)
             pending = self.d
         # only the last token needs logits

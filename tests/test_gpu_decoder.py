@@ -32,7 +32,7 @@ def test_rmsnorm_quant(ctx, M, H, with_delta):
     g = (1.0 + synth_normal(13, 0.1, (H,))).astype(np.float32)
     d_x, d_d, d_g = ctx.to_device(x), ctx.to_device(d), ctx.to_device(g)
     acts = ctx.alloc_acts(M, H)
-    check(ctx.lib.rbn_rmsnorm_quant_i8(ctx.handle, d_x.ptr, d_d.ptr if with_delta else None, d_g.ptr,
+    check(ctx.lib.rbn_rmsnorm_quant_i8(ctx.handle, d_x.ptr, d_d.ptr if with_delta else None, None, d_g.ptr,
                                        1e-5, M, H, acts[0].ptr, acts[1].ptr, acts[2].ptr))
     xin = (x + d).astype(np.float32) if with_delta else x
     y, q, s, rs = DM.rmsnorm_quant(xin, g, 1e-5)
@@ -47,6 +47,27 @@ def test_rmsnorm_quant(ctx, M, H, with_delta):
     assert (got_rs == got_q.astype(np.int32).sum(1)).all()
     if with_delta:   # the residual stream was updated in place, exactly
         assert (d_x.download(np.float32, M * H).reshape(M, H) == xin).all()
+
+
+@pytest.mark.parametrize("M,F", [(1, 6912), (3, 384), (2, 1000)])
+def test_rmsnorm_quant_with_swiglu_input(ctx, M, F):
+    gu = synth_normal(41 + M, 2.0, (M, 2 * F))
+    g = (1.0 + synth_normal(42, 0.1, (F,))).astype(np.float32)
+    d_gu, d_g = ctx.to_device(gu), ctx.to_device(g)
+    acts = ctx.alloc_acts(M, F)
+    check(ctx.lib.rbn_rmsnorm_quant_i8(ctx.handle, None, None, d_gu.ptr, d_g.ptr, 1e-5, M, F,
+                                       acts[0].ptr, acts[1].ptr, acts[2].ptr))
+    a, b = gu[:, :F], gu[:, F:]
+    h = ((a / (1.0 + np.exp(-a))) * b).astype(np.float32)
+    _, q, s, _ = DM.rmsnorm_quant(h, g, 1e-5)
+    pitch = ctx.act_pitch(F)
+    got_q = acts[0].download(np.int8, M * pitch).reshape(M, pitch)
+    diff = np.abs(got_q[:, :F].astype(np.int32) - q.astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 5e-3 and (got_q[:, F:] == 0).all()
+    assert close(acts[1].download(np.float32, M), s, rtol=1e-5)
+    with pytest.raises(_lib.RbnError):
+        check(ctx.lib.rbn_rmsnorm_quant_i8(ctx.handle, None, None, None, d_g.ptr, 1e-5, M, F,
+                                           acts[0].ptr, acts[1].ptr, acts[2].ptr))
 
 
 def test_embed_swiglu_argmax(ctx):
@@ -105,6 +126,18 @@ def test_rope_store_and_attention(ctx, M, pos0, heads):
         pr /= pr.sum(1, keepdims=True)
         want[m] = np.einsum("hn,hnd->hd", pr, gv[:, :n].astype(np.float64))
     assert close(out, want, rtol=2e-4, atol=2e-5)
+    if M == 1:   # the single-launch variant for decoding gives the same bits
+        kc2 = (np.random.default_rng(M * 1000 + pos0).normal(0, 1, (heads, max_seq, hd))).astype(np.float16)
+        vc2 = gv.copy()
+        vc2[:, pos, :] = 0
+        d_k2, d_v2, d_q2 = ctx.to_device(kc2.view(np.uint16)), ctx.to_device(vc2.view(np.uint16)), ctx.to_device(qkv)
+        d_out2 = ctx.alloc(4 * A)
+        check(ctx.lib.rbn_attention_decode_f16kv(ctx.handle, d_q2.ptr, d_pos.ptr, heads, hd, theta, d_k2.ptr,
+                                                 d_v2.ptr, max_seq, d_out2.ptr))
+        assert (d_out2.download(np.float32, A) == out.ravel()).all()
+        assert (d_k2.download(np.uint16, kc.size) == gk.view(np.uint16).ravel()).all()
+        assert (d_v2.download(np.uint16, vc.size) == gv.view(np.uint16).ravel()).all()
+        assert (d_q2.download(np.float32, 3 * A) == qkv.ravel()).all()
 
 
 def test_device_normal_generator(ctx):

@@ -171,12 +171,10 @@ __global__ __launch_bounds__(kBlock) void rope_kv_store_kernel(
 // One workgroup per (m, h); hd == 128.  Each wave takes every kWaves-th block of 64 keys:
 // scores with one key per lane (the key row is read as 16 x 16 bytes), online softmax,
 // then P.V with two dimensions per lane; the waves' (max, sum, out) meet through LDS.
-// FUSED (single token): the workgroup first rotates its head's q and k, writes k and v to
-// the cache (what rope_kv_store_kernel does) and then attends, one launch instead of two.
-template <int kWaves, bool FUSED>
+template <int kWaves>
 __global__ __launch_bounds__(kWaves * 64) void attention_kernel(
-    const float *__restrict__ qkv, const int32_t *__restrict__ pos0, int heads, float theta,
-    __half *__restrict__ kcache, __half *__restrict__ vcache, int max_seq,
+    const float *__restrict__ qkv, const int32_t *__restrict__ pos0, int heads,
+    const __half *__restrict__ kcache, const __half *__restrict__ vcache, int max_seq,
     float *__restrict__ out) {
     constexpr int hd = 128;
     __shared__ float s_q[hd];
@@ -190,53 +188,42 @@ __global__ __launch_bounds__(kWaves * 64) void attention_kernel(
     if (p >= max_seq) p = max_seq - 1;
     const int nkeys = p + 1;
     const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
-    if (FUSED) {
-        if (tid < hd / 2) {
-            const int i = tid, half = hd / 2;
-            const float freq = powf(theta, -2.0f * (float)i / (float)hd);
-            float sn, cs;
-            sincosf((float)p * freq, &sn, &cs);
-            const float *qh = qkv + (size_t)m * 3 * HD + h * hd, *kh_new = qh + HD, *vh_new = qh + 2 * HD;
-            const float q0 = qh[i], q1 = qh[i + half], k0 = kh_new[i], k1 = kh_new[i + half];
-            s_q[i] = (q0 * cs - q1 * sn) * scale;
-            s_q[i + half] = (q1 * cs + q0 * sn) * scale;
-            const size_t c = ((size_t)h * max_seq + p) * hd;
-            kcache[c + i] = __float2half_rn(k0 * cs - k1 * sn);
-            kcache[c + i + half] = __float2half_rn(k1 * cs + k0 * sn);
-            vcache[c + i] = __float2half_rn(vh_new[i]);
-            vcache[c + i + half] = __float2half_rn(vh_new[i + half]);
-        }
-    } else {
-        if (tid < hd) s_q[tid] = qkv[(size_t)m * 3 * HD + h * hd + tid] * scale;
-    }
-    __syncthreads();  // also makes the new cache row visible to the whole workgroup
+    if (tid < hd) s_q[tid] = qkv[(size_t)m * 3 * HD + h * hd + tid] * scale;
+    __syncthreads();
 
     const __half *kh = kcache + (size_t)h * max_seq * hd;
     const __half *vh = vcache + (size_t)h * max_seq * hd;
     float run_max = -INFINITY, run_sum = 0.0f, o0 = 0.0f, o1 = 0.0f;
     for (int t0 = wave * 64; t0 < nkeys; t0 += kWaves * 64) {
-        const int t = t0 + lane;
-        float s = -INFINITY;
-        if (t < nkeys) {
-            const uint4 *krow = reinterpret_cast<const uint4 *>(kh + (size_t)t * hd);
-            float acc = 0.0f;
+        // One round trip per block: the lane's key row (16 x 16 bytes) and its two columns
+        // of all 64 value rows are requested together; rows past the end repeat the last
+        // one and get probability 0.
+        const int last = nkeys - 1 - t0;  // >= 0
+        const int t = t0 + min(lane, last);
+        const uint4 *krow = reinterpret_cast<const uint4 *>(kh + (size_t)t * hd);
+        uint4 kr[hd / 8];
 #pragma unroll
-            for (int c = 0; c < hd / 8; ++c) {
-                const uint4 u = krow[c];
-                const __half2 *h2 = reinterpret_cast<const __half2 *>(&u);
+        for (int c = 0; c < hd / 8; ++c) kr[c] = krow[c];
+        __half2 vr[64];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float2 f = __half22float2(h2[e]);
-                    acc = fmaf(f.x, s_q[c * 8 + 2 * e], acc);
-                    acc = fmaf(f.y, s_q[c * 8 + 2 * e + 1], acc);
-                }
+        for (int j = 0; j < 64; ++j)
+            vr[j] = *reinterpret_cast<const __half2 *>(vh + (size_t)(t0 + min(j, last)) * hd + 2 * lane);
+        float acc = 0.0f;
+#pragma unroll
+        for (int c = 0; c < hd / 8; ++c) {
+            const __half2 *h2 = reinterpret_cast<const __half2 *>(&kr[c]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float2 f = __half22float2(h2[e]);
+                acc = fmaf(f.x, s_q[c * 8 + 2 * e], acc);
+                acc = fmaf(f.y, s_q[c * 8 + 2 * e + 1], acc);
             }
-            s = acc;
         }
+        const float s = lane <= last ? acc : -INFINITY;
         const float blk_max = wave_max_f(s);
         const float new_max = fmaxf(run_max, blk_max);
         const float corr = __expf(run_max - new_max);  // 0 on the first block
-        const float pr = t < nkeys ? __expf(s - new_max) : 0.0f;
+        const float pr = lane <= last ? __expf(s - new_max) : 0.0f;
         run_sum = run_sum * corr + wave_sum_f(pr);
         run_max = new_max;
         o0 *= corr;
@@ -244,21 +231,12 @@ __global__ __launch_bounds__(kWaves * 64) void attention_kernel(
         s_p[wave][lane] = pr;
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        // eight value rows per round, loads first; rows past the end repeat the last one
-        // with probability 0
-        const int last = nkeys - 1 - t0;
-        for (int j0 = 0; j0 <= min(63, last); j0 += 8) {
-            __half2 vr[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-                vr[u] = *reinterpret_cast<const __half2 *>(vh + (size_t)(t0 + min(j0 + u, last)) * hd + 2 * lane);
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const float pj = s_p[wave][j0 + u];  // 0 beyond the last key
-                const float2 v = __half22float2(vr[u]);
-                o0 = fmaf(pj, v.x, o0);
-                o1 = fmaf(pj, v.y, o1);
-            }
+        for (int j = 0; j < 64; ++j) {
+            const float pj = s_p[wave][j];
+            const float2 v = __half22float2(vr[j]);
+            o0 = fmaf(pj, v.x, o0);
+            o1 = fmaf(pj, v.y, o1);
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -283,6 +261,159 @@ __global__ __launch_bounds__(kWaves * 64) void attention_kernel(
         }
         out[(size_t)m * HD + h * hd + tid] = num / den;
     }
+}
+
+// Decoding one token: rotary embedding, cache store and attention in one launch, spread
+// over kSplits workgroups per head so that many CUs pull the cache at once.
+//  * Every workgroup rotates q (and the new k) itself; split 0 also writes the new k and v
+//    row to the cache.  The new row is taken from LDS, never re-read from memory.
+//  * Keys go to the 4 * kSplits waves of a head in blocks of 16; inside a block four lanes
+//    share a key (32 dimensions each) for the scores and every lane owns two dimensions
+//    for P.V, so a block is one round trip of 20 loads per lane.
+//  * The workgroups of a head publish (max, sum, out[128]) as device-scope stores, draw a
+//    ticket, and the last one combines and writes the result: no second launch, nobody waits.
+constexpr int kSplits = 8;
+constexpr int kPartial = 132;  // floats per partial: out[128], max, sum, padding
+__global__ __launch_bounds__(256) void attention_decode_kernel(
+    const float *__restrict__ qkv, const int32_t *__restrict__ pos, int heads, float theta,
+    __half *__restrict__ kcache, __half *__restrict__ vcache, int max_seq,
+    float *__restrict__ partials, unsigned *__restrict__ tickets, float *__restrict__ out) {
+    constexpr int hd = 128, half = 64;
+    __shared__ float s_q[hd], s_knew[hd], s_vnew[hd];
+    __shared__ float s_m[4], s_l[4];
+    __shared__ float s_o[4][hd];
+    __shared__ int s_last;
+    const int h = blockIdx.x / kSplits, sp = blockIdx.x - h * kSplits;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int HD = heads * hd;
+    int p = pos[0];
+    if (p >= max_seq) p = max_seq - 1;
+    const int nkeys = p + 1;
+    const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
+    if (tid < half) {
+        const int i = tid;
+        const float freq = powf(theta, -2.0f * (float)i / (float)hd);
+        float sn, cs;
+        sincosf((float)p * freq, &sn, &cs);
+        const float *qh = qkv + h * hd, *kn = qh + HD, *vn = qh + 2 * HD;
+        const float q0 = qh[i], q1 = qh[i + half], k0 = kn[i], k1 = kn[i + half];
+        s_q[i] = (q0 * cs - q1 * sn) * scale;
+        s_q[i + half] = (q1 * cs + q0 * sn) * scale;
+        const __half ka = __float2half_rn(k0 * cs - k1 * sn), kb = __float2half_rn(k1 * cs + k0 * sn);
+        const __half va = __float2half_rn(vn[i]), vb = __float2half_rn(vn[i + half]);
+        s_knew[i] = __half2float(ka);
+        s_knew[i + half] = __half2float(kb);
+        s_vnew[i] = __half2float(va);
+        s_vnew[i + half] = __half2float(vb);
+        if (sp == 0) {
+            const size_t c = ((size_t)h * max_seq + p) * hd;
+            kcache[c + i] = ka;
+            kcache[c + i + half] = kb;
+            vcache[c + i] = va;
+            vcache[c + i + half] = vb;
+        }
+    }
+    __syncthreads();
+
+    const __half *kh = kcache + (size_t)h * max_seq * hd;
+    const __half *vh = vcache + (size_t)h * max_seq * hd;
+    const int kidx = lane >> 2, sub = lane & 3;
+    float run_max = -INFINITY, run_sum = 0.0f, o0 = 0.0f, o1 = 0.0f;
+    for (int b = sp * 4 + wave; b * 16 < nkeys; b += 4 * kSplits) {
+        const int t0 = b * 16, last = nkeys - 1 - t0;  // last >= 0
+        const int t = t0 + min(kidx, last);
+        const uint4 *krow = reinterpret_cast<const uint4 *>(kh + (size_t)t * hd + sub * 32);
+        uint4 kr[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) kr[c] = krow[c];
+        __half2 vr[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+            vr[j] = *reinterpret_cast<const __half2 *>(vh + (size_t)(t0 + min(j, last)) * hd + 2 * lane);
+        float acc = 0.0f;
+        const bool fresh = t == p;  // the row this launch adds: take it from LDS
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const __half2 *h2 = reinterpret_cast<const __half2 *>(&kr[c]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int d = sub * 32 + c * 8 + 2 * e;
+                float2 f = __half22float2(h2[e]);
+                if (fresh) f = make_float2(s_knew[d], s_knew[d + 1]);
+                acc = fmaf(f.x, s_q[d], acc);
+                acc = fmaf(f.y, s_q[d + 1], acc);
+            }
+        }
+        acc += __shfl_xor(acc, 1);
+        acc += __shfl_xor(acc, 2);
+        const float s = kidx <= last ? acc : -INFINITY;
+        const float new_max = fmaxf(run_max, wave_max_f(s));
+        const float corr = __expf(run_max - new_max);  // 0 on the first block
+        const float pr = kidx <= last ? __expf(s - new_max) : 0.0f;
+        run_sum = run_sum * corr + wave_sum_f(sub == 0 ? pr : 0.0f);
+        run_max = new_max;
+        o0 *= corr;
+        o1 *= corr;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const float pj = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(pr), 4 * j));
+            // rows past the end were clamped loads of memory that may hold anything
+            float2 v = j <= last ? __half22float2(vr[j]) : make_float2(0.0f, 0.0f);
+            if (t0 + j == p) v = make_float2(s_vnew[2 * lane], s_vnew[2 * lane + 1]);
+            o0 = fmaf(pj, v.x, o0);
+            o1 = fmaf(pj, v.y, o1);
+        }
+    }
+    if (lane == 0) {
+        s_m[wave] = run_max;
+        s_l[wave] = run_sum;
+    }
+    s_o[wave][2 * lane] = o0;
+    s_o[wave][2 * lane + 1] = o1;
+    __syncthreads();
+    float *mine = partials + ((size_t)h * kSplits + sp) * kPartial;
+    if (tid < hd) {
+        float gmax = fmaxf(fmaxf(s_m[0], s_m[1]), fmaxf(s_m[2], s_m[3]));
+        float num = 0.0f, den = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float c = s_m[w] == -INFINITY ? 0.0f : __expf(s_m[w] - gmax);
+            num += c * s_o[w][tid];
+            den += c * s_l[w];
+        }
+        __hip_atomic_store(mine + tid, num, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) {
+            __hip_atomic_store(mine + hd, gmax, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(mine + hd + 1, den, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    // published once the stores have completed (vmcnt(0): this wave's; the barrier:
+    // everybody's); then one thread draws the ticket
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned ticket = atomicAdd(&tickets[h], 1u);
+        const int is_last = ticket == (unsigned)kSplits - 1;
+        if (is_last) atomicExch(&tickets[h], 0u);  // ready for the next launch
+        s_last = is_last;
+    }
+    __syncthreads();
+    if (!s_last || tid >= hd) return;
+    const float *all = partials + (size_t)h * kSplits * kPartial;
+    float ms[kSplits], gmax = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < kSplits; ++i) {
+        ms[i] = __hip_atomic_load(all + i * kPartial + hd, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        gmax = fmaxf(gmax, ms[i]);
+    }
+    float num = 0.0f, den = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kSplits; ++i) {
+        const float c = ms[i] == -INFINITY ? 0.0f : __expf(ms[i] - gmax);
+        num += c * __hip_atomic_load(all + i * kPartial + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        den += c * __hip_atomic_load(all + i * kPartial + hd + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    out[h * hd + tid] = num / den;
 }
 
 // h[m, f] = silu(gu[m, f]) * gu[m, F + f]
@@ -420,11 +551,11 @@ int rbn_attention_f16kv(rbn_ctx *ctx, const float *d_qkv, const int32_t *d_pos0,
                 "bad sizes in rbn_attention_f16kv");
     // a single token (decode) gets more waves per head: only `heads` workgroups run
     if (M == 1)
-        attention_kernel<16, false><<<dim3((unsigned)(M * heads)), dim3(16 * 64), 0, ctx->stream>>>(
-            d_qkv, d_pos0, (int)heads, 0.0f, (__half *)d_kcache, (__half *)d_vcache, (int)max_seq, d_out);
+        attention_kernel<8><<<dim3((unsigned)(M * heads)), dim3(8 * 64), 0, ctx->stream>>>(
+            d_qkv, d_pos0, (int)heads, (const __half *)d_kcache, (const __half *)d_vcache, (int)max_seq, d_out);
     else
-        attention_kernel<4, false><<<dim3((unsigned)(M * heads)), dim3(4 * 64), 0, ctx->stream>>>(
-            d_qkv, d_pos0, (int)heads, 0.0f, (__half *)d_kcache, (__half *)d_vcache, (int)max_seq, d_out);
+        attention_kernel<4><<<dim3((unsigned)(M * heads)), dim3(4 * 64), 0, ctx->stream>>>(
+            d_qkv, d_pos0, (int)heads, (const __half *)d_kcache, (const __half *)d_vcache, (int)max_seq, d_out);
     RBN_HIP(hipGetLastError());
     return RBN_OK;
 }
@@ -436,10 +567,14 @@ int rbn_attention_decode_f16kv(rbn_ctx *ctx, const float *d_qkv, const int32_t *
     RBN_REQUIRE(d_qkv && d_pos && d_kcache && d_vcache && d_out, "null pointer in rbn_attention_decode_f16kv");
     RBN_REQUIRE(head_dim == 128, "rbn_attention_decode_f16kv takes head_dim == 128 (got %llu)",
                 (unsigned long long)head_dim);
-    RBN_REQUIRE(heads > 0 && heads < 4096 && max_seq > 0 && max_seq < (1u << 24),
-                "bad sizes in rbn_attention_decode_f16kv");
-    attention_kernel<16, true><<<dim3((unsigned)heads), dim3(16 * 64), 0, ctx->stream>>>(
-        d_qkv, d_pos, (int)heads, theta, (__half *)d_kcache, (__half *)d_vcache, (int)max_seq, d_out);
+    // partial results and tickets live in the context's split workspace
+    RBN_REQUIRE(heads > 0 && heads <= RBN_SPLITK_GROUPS && max_seq > 0 && max_seq < (1u << 24),
+                "bad sizes in rbn_attention_decode_f16kv (heads <= %d)", RBN_SPLITK_GROUPS);
+    static_assert((size_t)RBN_SPLITK_GROUPS * kSplits * kPartial * 4 <= (size_t)RBN_SPLITK_TILES * 4096,
+                  "the attention partials must fit the split workspace");
+    attention_decode_kernel<<<dim3((unsigned)(heads * kSplits)), dim3(256), 0, ctx->stream>>>(
+        d_qkv, d_pos, (int)heads, theta, (__half *)d_kcache, (__half *)d_vcache, (int)max_seq,
+        (float *)ctx->splitk_partials, ctx->splitk_tickets, d_out);
     RBN_HIP(hipGetLastError());
     return RBN_OK;
 }

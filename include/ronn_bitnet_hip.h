@@ -219,6 +219,16 @@ int rbn_execute_ternary_matmul(rbn_ctx *ctx, const float *h_a, const float *h_b,
  * LLaMA / BitNet-b1.58 operations a decoder needs around it, so that a whole decode
  * step runs on the device and can be captured in a graph (positions and tokens are
  * read from device memory).  All row-major f32 unless said otherwise. */
+/* One-token BitLinear in one launch: RMSNorm of d_x [K] (or of silu(gate) * up when
+ * d_gate_up [2K] is given instead), per-token int8 quantisation as in
+ * rbn_rmsnorm_quant_i8, ternary GEMV, fused dequantisation, and
+ * out[n] = d_residual[n] + result when d_residual is given (it may be d_out itself).
+ * K % 16 == 0, K <= 8192.  The int8 codes can differ from rbn_rmsnorm_quant_i8's by one
+ * step where a value sits on a rounding boundary (different summation order). */
+int rbn_bitlinear_gemv_f32(rbn_ctx *ctx, const float *d_x, const float *d_gate_up,
+                           const float *d_gamma, float eps, const uint32_t *d_tiled,
+                           float w_scale, uint64_t K, uint64_t N, const float *d_residual,
+                           float *d_out);
 /* x[m,:] = table[tokens[m],:] (token ids clamped to [0, vocab)). */
 int rbn_embed_f32(rbn_ctx *ctx, const float *d_table, const int32_t *d_tokens, uint64_t M,
                   uint64_t H, uint64_t vocab, float *d_x);

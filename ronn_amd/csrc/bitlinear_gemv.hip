@@ -1,0 +1,334 @@
+// One-token BitLinear in a single launch: RMSNorm (optionally of SwiGLU(gate, up)), per-token
+// absmax int8 quantisation, ternary GEMV, fused dequantisation, optional residual add.
+//
+//   v      = x                         or  silu(gate) * up
+//   y      = (v * rsqrt(mean(v^2) + eps)) * gamma
+//   g      = max(max|y|, 1e-5);  q = clamp(rne(y * (127/g)), -128, 127);  s = g / 127
+//   out[n] = [residual[n] +] ((float)(sum_k q[k] * w[k,n]) * s) * w_scale
+//
+// The matmul and its epilogue are BitNetKernel::execute_ternary_matmul,
+// crates/ronn-providers/src/bitnet/kernels.rs:134-178 (epilogue order :168); the
+// normalisation and the int8 activations have no counterpart in the reference.
+//
+// Why one launch: at one token every kernel of a decoder layer is a few microseconds and
+// the gap between two dependent launches costs as much again, so the normalisation is
+// recomputed by every workgroup of the GEMV (the row is a few KiB in L2) while its first
+// weight loads are already in flight, instead of running as a launch of its own.  The GEMV
+// part is the decode kernel of gemv.hip: one wave per column quad, lanes split k, 4-bit
+// planes of the activations in LDS, v_dot8, DPP reduction.
+#include "common.hpp"
+
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int kMaxBlocksPerThread = 2;  // K <= 16 * 256 * 2 = 8192
+
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ int dpp_add(int v) {
+    return v + __builtin_amdgcn_update_dpp(0, v, CTRL, ROWMASK, 0xf, false);
+}
+// Sum over the 64 lanes of a wave; the total is valid in lane 63.
+__device__ __forceinline__ int wave_total_lane63(int v) {
+    v = dpp_add<0xB1, 0xf>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E, 0xf>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x124, 0xf>(v);  // row_ror:4
+    v = dpp_add<0x128, 0xf>(v);  // row_ror:8
+    v = dpp_add<0x142, 0xA>(v);  // row_bcast15
+    v = dpp_add<0x143, 0xC>(v);  // row_bcast31
+    return v;
+}
+__device__ __forceinline__ float wave_sum_f(float v) {
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+__device__ __forceinline__ float wave_max_f(float v) {
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
+    return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+// int8 x16 (natural k order) -> the four 4-bit planes that pair with the even/odd 2-bit
+// fields of a tiled weight word (see gemv.hip).
+__device__ __forceinline__ uint4 to_nibble_planes(uint4 a) {
+    uint4 p;
+    p.x = ((a.x >> 4) & 0x0F0F0F0Fu) | (a.z & 0xF0F0F0F0u);
+    p.y = (a.x & 0x0F0F0F0Fu) | ((a.z & 0x0F0F0F0Fu) << 4);
+    p.z = ((a.y >> 4) & 0x0F0F0F0Fu) | (a.w & 0xF0F0F0F0u);
+    p.w = (a.y & 0x0F0F0F0Fu) | ((a.w & 0x0F0F0F0Fu) << 4);
+    return p;
+}
+
+// KS waves per column quad, L weight loads in flight per lane and round, SWIGLU input.
+template <int KS, int L, bool SWIGLU>
+__global__ __launch_bounds__(kThreads) void bitlinear_gemv_kernel(
+    const float *__restrict__ x,        // [K], or gate|up [2K] with SWIGLU
+    const float *__restrict__ gamma,    // [K]
+    float eps, const uint4 *__restrict__ w4,  // [nquads][KB]
+    float w_scale, int K, int KB, int N, int nquads, const float *residual, float *out) {
+    constexpr int QPB = kWaves / KS;
+    extern __shared__ uint4 s_a[];  // KB staged activation blocks (4-bit planes)
+    __shared__ float s_red[kWaves];
+    __shared__ int s_redi[kWaves];
+    __shared__ int s_part[KS > 1 ? kWaves * 4 : 1];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int quad_local = wave / KS, slice = wave % KS;
+    int quad = blockIdx.x * QPB + quad_local;
+    const bool active = quad < nquads;
+    quad = active ? quad : nquads - 1;
+    const uint4 *wq = w4 + (size_t)quad * KB;
+    const int kreal = K >> 4;  // K % 16 == 0: blocks that hold activations (the rest is padding)
+
+    // this wave's k range
+    const int sl_len = (KB + KS - 1) / KS;
+    const int sl_lo = slice * sl_len;
+    const int sl_hi = min(sl_lo + sl_len, KB);
+
+    // (1) the row and the gains, (2) the first round of weights: all loads unconditional
+    // (indices clamped), back to back
+    float v[kMaxBlocksPerThread][16], gm[kMaxBlocksPerThread][16];
+#pragma unroll
+    for (int b = 0; b < kMaxBlocksPerThread; ++b) {
+        const int kb = min(tid + b * kThreads, kreal - 1);
+        const float4 *xr = reinterpret_cast<const float4 *>(x) + kb * 4;
+        const float4 *gr = reinterpret_cast<const float4 *>(gamma) + kb * 4;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const float4 a = xr[c], g4 = gr[c];
+            v[b][4 * c] = a.x, v[b][4 * c + 1] = a.y, v[b][4 * c + 2] = a.z, v[b][4 * c + 3] = a.w;
+            gm[b][4 * c] = g4.x, gm[b][4 * c + 1] = g4.y, gm[b][4 * c + 2] = g4.z, gm[b][4 * c + 3] = g4.w;
+        }
+        if (SWIGLU) {
+            const float4 *ur = reinterpret_cast<const float4 *>(x + K) + kb * 4;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const float4 u = ur[c];
+                const float uu[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float g = v[b][4 * c + e];
+                    v[b][4 * c + e] = (g / (1.0f + __expf(-g))) * uu[e];
+                }
+            }
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    uint4 w[L];
+#pragma unroll
+    for (int it = 0; it < L; ++it) {
+        const int kb = sl_lo + it * 64 + lane;
+        w[it] = wq[kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // normalise and quantise (every workgroup computes the same values in the same order)
+    float ss = 0.0f;
+#pragma unroll
+    for (int b = 0; b < kMaxBlocksPerThread; ++b) {
+        const bool mine = tid + b * kThreads < kreal;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            v[b][e] = mine ? v[b][e] : 0.0f;
+            ss += v[b][e] * v[b][e];
+        }
+    }
+    ss = wave_sum_f(ss);
+    if (lane == 0) s_red[wave] = ss;
+    __syncthreads();
+    ss = (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
+    const float inv_rms = 1.0f / sqrtf(ss / (float)K + eps);
+    float amax = 0.0f;
+#pragma unroll
+    for (int b = 0; b < kMaxBlocksPerThread; ++b)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            v[b][e] = (v[b][e] * inv_rms) * gm[b][e];
+            amax = fmaxf(amax, fabsf(v[b][e]));
+        }
+    amax = wave_max_f(amax);
+    __syncthreads();
+    if (lane == 0) s_red[wave] = amax;
+    __syncthreads();
+    const float gmax = fmaxf(fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3])), 1e-5f);
+    const float inv = 127.0f / gmax;
+    const float act_scale = gmax / 127.0f;
+    int qsum = 0;
+#pragma unroll
+    for (int b = 0; b < kMaxBlocksPerThread; ++b) {
+        const int kb = tid + b * kThreads;
+        uint32_t pk[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float r = rintf(v[b][4 * c + e] * inv);  // round half to even
+                r = fminf(fmaxf(r, -128.0f), 127.0f);
+                const int qi = (int)r;
+                qsum += qi;
+                word |= (uint32_t)(qi & 0xff) << (8 * e);
+            }
+            pk[c] = word;
+        }
+        if (kb < KB) s_a[kb] = to_nibble_planes(make_uint4(pk[0], pk[1], pk[2], pk[3]));  // zeros in the padding
+    }
+    qsum = wave_sum_i(qsum);
+    if (lane == 0) s_redi[wave] = qsum;
+    __syncthreads();
+    const int rowsum = (s_redi[0] + s_redi[1]) + (s_redi[2] + s_redi[3]);
+
+    int hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
+    auto consume = [&](const uint4(&wr)[L], int r0) {
+#pragma unroll
+        for (int it = 0; it < L; ++it) {
+            const int kb = r0 + it * 64 + lane;
+            const uint32_t keep = kb < sl_hi ? 0x33333333u : 0u;
+            const uint4 a = s_a[min(kb, sl_hi - 1)];
+            const uint32_t ww[4] = {wr[it].x, wr[it].y, wr[it].z, wr[it].w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t ev = ww[c] & keep, od = (ww[c] >> 2) & keep;
+                hi[c] = __builtin_amdgcn_sdot8((int)a.x, (int)ev, hi[c], false);
+                lo[c] = (int)__builtin_amdgcn_udot8(a.y, ev, (uint32_t)lo[c], false);
+                hi[c] = __builtin_amdgcn_sdot8((int)a.z, (int)od, hi[c], false);
+                lo[c] = (int)__builtin_amdgcn_udot8(a.w, od, (uint32_t)lo[c], false);
+            }
+        }
+    };
+    int r0 = sl_lo;
+    while (r0 + 64 * L < sl_hi) {
+        uint4 wn[L];
+#pragma unroll
+        for (int it = 0; it < L; ++it) {
+            const int kb = r0 + 64 * L + it * 64 + lane;
+            wn[it] = wq[kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)];
+        }
+        consume(w, r0);
+#pragma unroll
+        for (int it = 0; it < L; ++it) w[it] = wn[it];
+        r0 += 64 * L;
+    }
+    if (r0 < sl_hi) consume(w, r0);
+
+    int tot[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) tot[c] = wave_total_lane63(hi[c] * 16 + lo[c]);
+
+    auto finish = [&](int n, int total) {
+        total -= rowsum;
+        float r = (float)total * act_scale;  // kernels.rs:168, left to right
+        r = r * w_scale;
+        if (residual) r = residual[n] + r;
+        out[n] = r;
+    };
+    if (KS == 1) {
+        if (lane == 63 && active) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int n = quad * 4 + c;
+                if (n < N) finish(n, tot[c]);
+            }
+        }
+    } else {
+        if (lane == 63) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) s_part[wave * 4 + c] = tot[c];
+        }
+        __syncthreads();
+        if (tid < QPB * 4) {
+            const int ql = tid >> 2, c = tid & 3;
+            const int qd = blockIdx.x * QPB + ql, n = qd * 4 + c;
+            if (qd < nquads && n < N) {
+                int total = 0;
+#pragma unroll
+                for (int s = 0; s < KS; ++s) total += s_part[(ql * KS + s) * 4 + c];
+                finish(n, total);
+            }
+        }
+    }
+}
+
+struct Args {
+    const float *x, *gamma;
+    float eps;
+    const uint4 *w4;
+    float w_scale;
+    int K, KB, N, nquads;
+    const float *residual;
+    float *out;
+};
+
+template <int KS, int L, bool SWIGLU>
+void launch(hipStream_t stream, const Args &a) {
+    constexpr int QPB = kWaves / KS;
+    dim3 grid((unsigned)((a.nquads + QPB - 1) / QPB));
+    bitlinear_gemv_kernel<KS, L, SWIGLU><<<grid, dim3(kThreads), (size_t)a.KB * 16, stream>>>(
+        a.x, a.gamma, a.eps, a.w4, a.w_scale, a.K, a.KB, a.N, a.nquads, a.residual, a.out);
+}
+
+template <int KS, bool SWIGLU>
+void launch_l(hipStream_t stream, const Args &a) {
+    const int loads = ((a.KB + KS - 1) / KS + 63) / 64;  // per lane, to cover a wave's share
+    if (loads <= 1)
+        launch<KS, 1, SWIGLU>(stream, a);
+    else if (loads <= 2)
+        launch<KS, 2, SWIGLU>(stream, a);
+    else
+        launch<KS, 4, SWIGLU>(stream, a);
+}
+
+template <bool SWIGLU>
+void launch_ks(hipStream_t stream, const Args &a) {
+    // waves per quad: as in the plain GEMV, enough wavefronts for the chip without
+    // shrinking a wave's share of k below one round
+    int ks = 1;
+    while (ks < 4 && (long long)a.nquads * ks < 2048 && a.KB / (ks * 2) >= 128) ks *= 2;
+    if (ks == 4)
+        launch_l<4, SWIGLU>(stream, a);
+    else if (ks == 2)
+        launch_l<2, SWIGLU>(stream, a);
+    else
+        launch_l<1, SWIGLU>(stream, a);
+}
+
+}  // namespace
+
+extern "C" int rbn_bitlinear_gemv_f32(rbn_ctx *ctx, const float *d_x, const float *d_gate_up,
+                                      const float *d_gamma, float eps, const uint32_t *d_tiled,
+                                      float w_scale, uint64_t K, uint64_t N, const float *d_residual,
+                                      float *d_out) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE((d_x != nullptr) != (d_gate_up != nullptr),
+                "rbn_bitlinear_gemv_f32 takes either d_x or d_gate_up");
+    RBN_REQUIRE(d_gamma && d_tiled && d_out, "null pointer in rbn_bitlinear_gemv_f32");
+    RBN_REQUIRE(K >= 16 && K % 16 == 0 && K <= 16ull * kThreads * kMaxBlocksPerThread,
+                "rbn_bitlinear_gemv_f32 takes K %% 16 == 0, 16 <= K <= %d (got %llu)",
+                16 * kThreads * kMaxBlocksPerThread, (unsigned long long)K);
+    RBN_REQUIRE(N > 0 && N <= (1ull << 30), "bad N in rbn_bitlinear_gemv_f32");
+    const float *src = d_x ? d_x : d_gate_up;
+    RBN_REQUIRE((((uintptr_t)src | (uintptr_t)d_gamma | (uintptr_t)d_tiled) & 15u) == 0,
+                "inputs must be 16-byte aligned");
+    Args a;
+    a.x = src;
+    a.gamma = d_gamma;
+    a.eps = eps;
+    a.w4 = (const uint4 *)d_tiled;
+    a.w_scale = w_scale;
+    a.K = (int)K;
+    a.KB = (int)(rbn_kpad(K) / 16);
+    a.N = (int)N;
+    a.nquads = (int)(rbn_npad(N) / 4);
+    a.residual = d_residual;
+    a.out = d_out;
+    if (d_gate_up)
+        launch_ks<true>(ctx->stream, a);
+    else
+        launch_ks<false>(ctx->stream, a);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}

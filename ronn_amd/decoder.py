@@ -163,6 +163,33 @@ class BitNetDecoder:
     def _linear(self, lin: _Linear, M: int, out: DeviceBuffer):
         self.ctx.matmul(self.acts, lin.tiled, lin.scale, M, lin.K, lin.N, d_out=out)
 
+    def _bitlinear1(self, lin: _Linear, gamma: DeviceBuffer, out: DeviceBuffer, x=None, gate_up=None,
+                    residual=None, row0: int = 0):
+        """One token: norm + quant + GEMV (+ residual) in one launch."""
+        off = 4 * row0 * lin.K
+        check(self.lib.rbn_bitlinear_gemv_f32(
+            self.ctx.handle, (x.ptr + off) if x is not None else None,
+            gate_up.ptr if gate_up is not None else None, gamma.ptr, self.cfg.eps, lin.tiled.ptr, lin.scale,
+            lin.K, lin.N, residual.ptr if residual is not None else None, out.ptr))
+
+    def forward_one(self):
+        """forward(1) with five launches per layer: every BitLinear is one kernel, the
+        residual additions ride on the o and down projections."""
+        cfg, lib, hnd = self.cfg, self.lib, self.ctx.handle
+        check(lib.rbn_embed_f32(hnd, self.embed.ptr, self.tokens.ptr, 1, cfg.hidden, cfg.vocab, self.x.ptr))
+        for i, b in enumerate(self.blocks):
+            self._bitlinear1(b["wqkv"], b["g_attn"], self.qkv, x=self.x)
+            check(lib.rbn_attention_decode_f16kv(hnd, self.qkv.ptr, self.pos.ptr, cfg.heads, cfg.head_dim,
+                                                 cfg.rope_theta, self.kcache[i].ptr, self.vcache[i].ptr,
+                                                 cfg.max_seq, self.att.ptr))
+            self._bitlinear1(b["wo"], b["g_attn_sub"], self.x, x=self.att, residual=self.x)
+            self._bitlinear1(b["wgu"], b["g_ffn"], self.gu, x=self.x)
+            self._bitlinear1(b["wdown"], b["g_ffn_sub"], self.x, gate_up=self.gu, residual=self.x)
+        self._bitlinear1(self.lm_head, self.g_final, self.logits, x=self.x)
+        check(lib.rbn_add_i32(hnd, self.pos.ptr, 1))
+        check(lib.rbn_argmax_f32(hnd, self.logits.ptr, cfg.vocab, self.tokens.ptr, self.history.ptr,
+                                 self.pos.ptr))
+
     def forward(self, M: int):
         """Tokens self.tokens[0:M] at positions *pos .. *pos+M-1; leaves the logits of the
         last token in self.logits and its arg-max in self.tokens[0] and the history."""
@@ -193,7 +220,10 @@ class BitNetDecoder:
             self._norm_quant(None, None, b["g_ffn_sub"], M, F, gate_up=self.gu)   # SwiGLU fused in
             self._linear(b["wdown"], M, self.d)
             pending = self.d
-        # only the last token needs logits
+        # only the last token needs logits; the pending residual is added for every row, so
+        # that self.x is the complete residual stream
+        if M > 1:
+            self._norm_quant(self.x, pending, self.g_final, M - 1, H)
         self._norm_quant(self.x, pending, self.g_final, 1, H, row0=M - 1)
         self._linear(self.lm_head, 1, self.logits)
         check(lib.rbn_add_i32(hnd, self.pos.ptr, M))
@@ -213,7 +243,7 @@ class BitNetDecoder:
     def capture_decode_step(self):
         if self._graph is None:
             self.ctx.graph_begin()
-            self.forward(1)
+            self.forward_one()
             self._graph = self.ctx.graph_end()
         return self._graph
 
@@ -226,7 +256,7 @@ class BitNetDecoder:
             if g is not None:
                 self.ctx.graph_launch(g)
             else:
-                self.forward(1)
+                self.forward_one()
         self.ctx.sync()
         dt = time.perf_counter() - t0
         return self.generated(n_tokens + 1)[1:], dt

@@ -70,6 +70,41 @@ def test_rmsnorm_quant_with_swiglu_input(ctx, M, F):
                                            acts[0].ptr, acts[1].ptr, acts[2].ptr))
 
 
+@pytest.mark.parametrize("K,N", [(2560, 7680), (2560, 2560), (6912, 2560), (2560, 13824), (256, 1000), (8192, 96), (16, 4)])
+@pytest.mark.parametrize("mode", ["plain", "residual", "swiglu"])
+def test_bitlinear_gemv_single_launch(ctx, K, N, mode):
+    """RMSNorm + quant + ternary GEMV (+ SwiGLU on the way in, + residual) in one launch
+    against the numpy model; the BitLinear inside goes through the CPU oracle."""
+    from util import oracle_weights, exact_int_matmul, epilogue
+    w = synth_normal(51 + K, 0.02, (K, N))
+    g = (1.0 + synth_normal(52, 0.1, (K,))).astype(np.float32)
+    res = synth_normal(53, 1.0, (N,))
+    if mode == "swiglu":
+        gu = synth_normal(54 + N, 2.0, (1, 2 * K))
+        a, b = gu[:, :K], gu[:, K:]
+        v = ((a / (1.0 + np.exp(-a))) * b).astype(np.float32)
+    else:
+        v = synth_normal(55 + N, 1.0, (1, K))
+    d_w = ctx.to_device(w)
+    d_p, w_scale, _, _ = ctx.quantize_ternary(d_w, w.size)
+    d_t = ctx.tile_weights(d_p, K, N)
+    d_in = ctx.to_device(gu if mode == "swiglu" else v)
+    d_g, d_out = ctx.to_device(g), ctx.to_device(res.copy())
+    check(ctx.lib.rbn_bitlinear_gemv_f32(
+        ctx.handle, None if mode == "swiglu" else d_in.ptr, d_in.ptr if mode == "swiglu" else None, d_g.ptr,
+        1e-5, d_t.ptr, float(w_scale), K, N, d_out.ptr if mode == "residual" else None, d_out.ptr))
+    got = d_out.download(np.float32, N)
+    _, q, s, _ = DM.rmsnorm_quant(v, g, 1e-5)
+    t, vals = oracle_weights(w)
+    want = epilogue(exact_int_matmul(q, vals), s, t.scale)[0]
+    if mode == "residual":
+        want = (res + want).astype(np.float32)
+    # a code that flips by one step moves an output by one quantisation step of the product
+    step = float(s[0]) * float(t.scale)
+    assert np.abs(got - want).max() <= 4 * step + 1e-6 * np.abs(want).max()
+    assert (got == want).mean() > 0.5 or K <= 16 or mode == "swiglu"
+
+
 def test_embed_swiglu_argmax(ctx):
     V, H, M, F = 1000, 256, 7, 300
     table = synth_normal(21, 1.0, (V, H))

@@ -96,6 +96,22 @@ int rbp_ternary_packed(rbp_ternary *t, uint8_t *h_out, uint64_t capacity);
 int rbp_ternary_get_value(rbp_ternary *t, uint64_t index);
 int rbp_dequantize_ternary(rbp_provider *p, rbp_ternary *t, float *h_out, uint64_t capacity);
 
+/* Packed-weight files: ternarisation as a one-time offline step.  The reference has
+ * TernaryTensor's fields (quantization.rs:249-260) and no serialisation; the format is
+ * this build's ("RBNTERN1", version, shape, scale, threshold, packed bytes in the
+ * reference's layout, CRC-32; see csrc/host/bitnet_provider.hpp).  None of these
+ * needs a GPU. */
+int rbp_ternary_from_parts(const uint8_t *h_packed, uint64_t packed_bytes, const uint64_t *shape,
+                           int ndim, float scale, float threshold, rbp_ternary **out);
+int rbp_ternary_shape(rbp_ternary *t, uint64_t shape[8], int *ndim);
+int rbp_ternary_save(rbp_ternary *t, const char *path);
+int rbp_ternary_load(const char *path, rbp_ternary **out);
+/* TernaryMatMul with weights that are already ternarised: A [m,k] f32 (host) is
+ * quantised as rbp_kernel_execute does, B [k,n] comes from `w`. */
+int rbp_kernel_execute_prepacked(rbp_kernel *k, const float *h_a, const uint64_t *shape_a, int ndim_a,
+                                 rbp_ternary *w, float *h_out, uint64_t out_capacity,
+                                 uint64_t out_shape[2]);
+
 #ifdef __cplusplus
 }
 #endif

@@ -235,6 +235,11 @@ PROVIDER_SIGNATURES = {
     "rbp_ternary_packed": (C.c_int, [_vp, _vp, _u64]),
     "rbp_ternary_get_value": (C.c_int, [_vp, _u64]),
     "rbp_dequantize_ternary": (C.c_int, [_vp, _vp, _vp, _u64]),
+    "rbp_ternary_from_parts": (C.c_int, [_vp, _u64, _u64p, C.c_int, C.c_float, C.c_float, C.POINTER(_vp)]),
+    "rbp_ternary_shape": (C.c_int, [_vp, _u64p, C.POINTER(C.c_int)]),
+    "rbp_ternary_save": (C.c_int, [_vp, C.c_char_p]),
+    "rbp_ternary_load": (C.c_int, [C.c_char_p, C.POINTER(_vp)]),
+    "rbp_kernel_execute_prepacked": (C.c_int, [_vp, _vp, _u64p, C.c_int, _vp, _vp, _u64, _u64p]),
 }
 
 _bound = None
@@ -279,6 +284,28 @@ class TernaryTensor:
         self.packed_data = np.zeros(m.value, dtype=np.uint8)
         if m.value:
             _check(_api().rbp_ternary_packed(handle, self.packed_data.ctypes.data, m.value))
+
+    @classmethod
+    def from_parts(cls, packed_data, shape, scale, threshold) -> "TernaryTensor":
+        """A tensor from fields produced elsewhere (e.g. an offline quantiser); checked
+        against the invariants of quantize_ternary.  Needs no GPU."""
+        packed = np.ascontiguousarray(packed_data, dtype=np.uint8)
+        h = _vp()
+        _check(_api().rbp_ternary_from_parts(packed.ctypes.data, packed.size, _shape_arg(shape), len(shape),
+                                             float(scale), float(threshold), C.byref(h)))
+        return cls(h.value, shape)
+
+    def save(self, path: str):
+        """Writes the packed-weight file (format: csrc/host/bitnet_provider.hpp)."""
+        _check(_api().rbp_ternary_save(self._h, str(path).encode()))
+
+    @classmethod
+    def load(cls, path: str) -> "TernaryTensor":
+        h = _vp()
+        _check(_api().rbp_ternary_load(str(path).encode(), C.byref(h)))
+        shape, ndim = (C.c_uint64 * 8)(), C.c_int()
+        _check(_api().rbp_ternary_shape(h.value, shape, C.byref(ndim)))
+        return cls(h.value, [int(shape[i]) for i in range(ndim.value)])
 
     def memory_size(self) -> int:
         return self._memory_size
@@ -343,6 +370,18 @@ class BitNetKernel:
                                          cap, out_shape))
         m, nn = out_shape[0], out_shape[1]
         return [Tensor(out[:m * nn].reshape(m, nn), DataType.F32, TensorLayout.RowMajor)]
+
+    def execute_prepacked(self, a: Tensor, weights: "TernaryTensor") -> Tensor:
+        """TernaryMatMul with weights that are already ternarised (a loaded weight file)."""
+        arr = np.ascontiguousarray(a.to_vec(), dtype=np.float32)
+        cap = max(1, a.shape()[0] * (weights.shape[1] if len(weights.shape) == 2 else 1))
+        out = np.empty(cap, dtype=np.float32)
+        out_shape = (C.c_uint64 * 2)()
+        _check(_api().rbp_kernel_execute_prepacked(self._h, arr.ctypes.data, _shape_arg(a.shape()),
+                                                   len(a.shape()), weights._h, out.ctypes.data, cap,
+                                                   out_shape))
+        m, nn = out_shape[0], out_shape[1]
+        return Tensor(out[:m * nn].reshape(m, nn), DataType.F32, TensorLayout.RowMajor)
 
     def get_performance_stats(self) -> KernelStats:
         c, a, lo, hi = C.c_uint64(), C.c_double(), C.c_double(), C.c_double()

@@ -1,6 +1,8 @@
 // Implementation of the MI355X BitNet execution provider (host side); see the header.
 #include "bitnet_provider.hpp"
 
+#include <cstdio>
+
 #include <chrono>
 #include <cstring>
 #include <sstream>
@@ -178,47 +180,63 @@ Tensor BitNetKernel::execute_ternary_matmul(const Tensor &a, const Tensor &b) {
     if (m == 0 || n == 0 || k == 0)
         return Tensor::from_data(std::vector<float>(m * n, 0.0f), {m, n}, DataType::F32,
                                  TensorLayout::RowMajor);
-    rbn_ctx *ctx = device_->ctx();
-
     // weights: ternarise + tile once per distinct content (kernels.rs:278 does it per call)
-    CachedWeights w;
     bool owned = false;
-    uint64_t key = 0;
-    if (cache_weights_) {
-        key = hash_floats(b.to_vec(), b.shape());
-        auto it = weight_cache_.find(key);
-        if (it != weight_cache_.end()) w = it->second;
-    }
-    if (!w.d_tiled) {
-        DBuf d_b(ctx, k * n * 4), d_p(ctx, rbn_packed_capacity(k * n));
-        DBuf d_t(ctx, rbn_tiled_bytes(k, n));
-        float thr = 0.0f;
-        check(rbn_h2d(ctx, d_b.p, b.to_vec().data(), k * n * 4), "rbn_h2d");
-        check(rbn_quantize_ternary(ctx, (const float *)d_b.p, k * n, sum_mode_, (uint8_t *)d_p.p,
-                                   &w.scale, &thr, nullptr),
-              "rbn_quantize_ternary");
-        check(rbn_tile_weights(ctx, (const uint8_t *)d_p.p, k, n, (uint32_t *)d_t.p),
-              "rbn_tile_weights");
-        w.bytes = rbn_tiled_bytes(k, n);
-        w.d_tiled = d_t.release();
-        if (cache_weights_ && cache_bytes_ + w.bytes <= max_cache_bytes_) {
-            weight_cache_[key] = w;
-            cache_bytes_ += w.bytes;
-            memory_usage_.current_bytes = cache_bytes_;
-            if (cache_bytes_ > memory_usage_.peak_bytes) memory_usage_.peak_bytes = cache_bytes_;
-            memory_usage_.allocation_count += 1;
-        } else {
-            owned = true;
-        }
-    }
+    const uint64_t key = cache_weights_ ? hash_floats(b.to_vec(), b.shape()) : 0;
+    CachedWeights w = tiled_weights(key, k, n, nullptr, b.to_vec().data(), 1.0f, &owned);
     struct Release {
         rbn_ctx *c;
         void *p;
         ~Release() {
             if (p) rbn_free(c, p);
         }
-    } release{ctx, owned ? w.d_tiled : nullptr};
+    } release{device_->ctx(), owned ? w.d_tiled : nullptr};
+    return multiply(a, m, k, n, w.d_tiled, w.scale);
+}
 
+BitNetKernel::CachedWeights BitNetKernel::tiled_weights(uint64_t key, size_t k, size_t n,
+                                                        const uint8_t *h_packed, const float *h_f32,
+                                                        float scale, bool *owned) {
+    rbn_ctx *ctx = device_->ctx();
+    CachedWeights w;
+    *owned = false;
+    if (cache_weights_) {
+        auto it = weight_cache_.find(key);
+        if (it != weight_cache_.end()) return it->second;
+    }
+    DBuf d_p(ctx, rbn_packed_capacity(k * n));
+    DBuf d_t(ctx, rbn_tiled_bytes(k, n));
+    if (h_f32) {
+        DBuf d_b(ctx, k * n * 4);
+        float thr = 0.0f;
+        check(rbn_h2d(ctx, d_b.p, h_f32, k * n * 4), "rbn_h2d");
+        check(rbn_quantize_ternary(ctx, (const float *)d_b.p, k * n, sum_mode_, (uint8_t *)d_p.p,
+                                   &w.scale, &thr, nullptr),
+              "rbn_quantize_ternary");
+    } else {
+        check(rbn_fill_u8(ctx, d_p.p, 0x55, rbn_packed_capacity(k * n)), "rbn_fill_u8");  // code 01 = 0
+        check(rbn_h2d(ctx, d_p.p, h_packed, (k * n + 3) / 4), "rbn_h2d");
+        w.scale = scale;
+    }
+    check(rbn_tile_weights(ctx, (const uint8_t *)d_p.p, k, n, (uint32_t *)d_t.p), "rbn_tile_weights");
+    check(rbn_sync(ctx), "rbn_sync");
+    w.bytes = rbn_tiled_bytes(k, n);
+    w.d_tiled = d_t.release();
+    if (cache_weights_ && cache_bytes_ + w.bytes <= max_cache_bytes_) {
+        weight_cache_[key] = w;
+        cache_bytes_ += w.bytes;
+        memory_usage_.current_bytes = cache_bytes_;
+        if (cache_bytes_ > memory_usage_.peak_bytes) memory_usage_.peak_bytes = cache_bytes_;
+        memory_usage_.allocation_count += 1;
+    } else {
+        *owned = true;
+    }
+    return w;
+}
+
+Tensor BitNetKernel::multiply(const Tensor &a, size_t m, size_t k, size_t n, const void *d_tiled,
+                              float w_scale) {
+    rbn_ctx *ctx = device_->ctx();
     // activations (kernels.rs:277): per-tensor ternary as the reference, or per-token int8
     DBuf d_a(ctx, m * k * 4), d_q(ctx, m * rbn_act_pitch(k)), d_s(ctx, m * 4), d_r(ctx, m * 4);
     DBuf d_o(ctx, m * n * 4);
@@ -234,11 +252,149 @@ Tensor BitNetKernel::execute_ternary_matmul(const Tensor &a, const Tensor &b) {
     }
     // kernels.rs:280-281 and the epilogue of :168
     check(rbn_matmul_t2_i8(ctx, (const int8_t *)d_q.p, (const float *)d_s.p, (const int32_t *)d_r.p,
-                           (const uint32_t *)w.d_tiled, w.scale, m, k, n, nullptr, (float *)d_o.p),
+                           (const uint32_t *)d_tiled, w_scale, m, k, n, nullptr, (float *)d_o.p),
           "rbn_matmul_t2_i8");
     std::vector<float> result(m * n);
     check(rbn_d2h(ctx, result.data(), d_o.p, m * n * 4), "rbn_d2h");
     return Tensor::from_data(std::move(result), {m, n}, DataType::F32, TensorLayout::RowMajor);
+}
+
+Tensor BitNetKernel::execute_prepacked(const Tensor &a, const TernaryTensor &w) {
+    const auto start = std::chrono::steady_clock::now();
+    std::lock_guard<std::mutex> guard(lock_);
+    if (operation_.kind != BitNetOperation::TernaryMatMul)
+        throw Error("execute_prepacked needs a TernaryMatMul kernel");
+    require_f32(a);
+    validate_ternary_tensor(w);
+    if (a.shape().size() != 2 || w.shape.size() != 2 || a.shape()[1] != w.shape[0])
+        throw Error("Matrix dimension mismatch: A=" + shape_str(a.shape()) + ", B=" + shape_str(w.shape) +
+                    ", expected A=[m,k], B=[k,n]");
+    const size_t m = a.shape()[0], k = a.shape()[1], n = w.shape[1];
+    if ((operation_.m || operation_.n || operation_.k) &&
+        (operation_.m != m || operation_.n != n || operation_.k != k))
+        throw Error("Matrix dimension mismatch: the kernel was compiled for other dimensions");
+    if (m == 0 || n == 0 || k == 0)
+        return Tensor::from_data(std::vector<float>(m * n, 0.0f), {m, n}, DataType::F32,
+                                 TensorLayout::RowMajor);
+    // cache key: content of the packed bytes, shape and scale
+    uint64_t key = 0;
+    if (cache_weights_) {
+        std::vector<float> as_f((w.packed_data.size() + 3) / 4 + 1, 0.0f);
+        std::memcpy(as_f.data(), w.packed_data.data(), w.packed_data.size());
+        std::memcpy(&as_f.back(), &w.scale, 4);
+        key = hash_floats(as_f, w.shape) ^ 0x5bd1e9955bd1e995ull;
+    }
+    bool owned = false;
+    CachedWeights cw = tiled_weights(key, k, n, w.packed_data.data(), nullptr, w.scale, &owned);
+    struct Release {
+        rbn_ctx *c;
+        void *p;
+        ~Release() {
+            if (p) rbn_free(c, p);
+        }
+    } release{device_->ctx(), owned ? cw.d_tiled : nullptr};
+    Tensor out = multiply(a, m, k, n, cw.d_tiled, cw.scale);
+    update_stats(std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - start).count());
+    return out;
+}
+
+// ---- packed-weight file ----------------------------------------------------------------------
+namespace {
+uint32_t crc32_ieee(const uint8_t *p, size_t n, uint32_t crc = 0) {
+    static uint32_t table[256];
+    static bool ready = false;
+    if (!ready) {
+        for (uint32_t i = 0; i < 256; ++i) {
+            uint32_t c = i;
+            for (int j = 0; j < 8; ++j) c = (c & 1) ? 0xEDB88320u ^ (c >> 1) : c >> 1;
+            table[i] = c;
+        }
+        ready = true;
+    }
+    crc = ~crc;
+    for (size_t i = 0; i < n; ++i) crc = table[(crc ^ p[i]) & 0xff] ^ (crc >> 8);
+    return ~crc;
+}
+template <typename T>
+void put(std::vector<uint8_t> &out, T v) {
+    uint8_t b[sizeof(T)];
+    std::memcpy(b, &v, sizeof(T));  // the build targets little-endian hosts only
+    out.insert(out.end(), b, b + sizeof(T));
+}
+template <typename T>
+T get(const std::vector<uint8_t> &in, size_t &off) {
+    if (off + sizeof(T) > in.size()) throw Error("packed-weight file is truncated");
+    T v;
+    std::memcpy(&v, in.data() + off, sizeof(T));
+    off += sizeof(T);
+    return v;
+}
+const char kMagic[8] = {'R', 'B', 'N', 'T', 'E', 'R', 'N', '1'};
+}  // namespace
+
+void validate_ternary_tensor(const TernaryTensor &t) {
+    size_t n = 1;
+    for (size_t d : t.shape) n *= d;
+    if (t.shape.empty()) n = t.element_count;
+    if (n != t.element_count) throw Error("ternary tensor: shape does not match element_count");
+    if (t.packed_data.size() != (t.element_count + 3) / 4)
+        throw Error("ternary tensor: packed size is not ceil(element_count / 4)");
+    if (t.element_count % 4 != 0 && !t.packed_data.empty()) {
+        const unsigned used = (unsigned)(t.element_count % 4) * 2;
+        if (t.packed_data.back() >> used) throw Error("ternary tensor: tail bits are not zero");
+    }
+}
+
+void save_ternary_tensor(const TernaryTensor &t, const std::string &path) {
+    validate_ternary_tensor(t);
+    if (t.shape.size() > 8) throw Error("ternary tensor: more than 8 dimensions");
+    std::vector<uint8_t> out;
+    out.reserve(64 + t.packed_data.size());
+    out.insert(out.end(), kMagic, kMagic + 8);
+    put<uint32_t>(out, 1);
+    put<uint32_t>(out, (uint32_t)t.shape.size());
+    put<uint64_t>(out, (uint64_t)t.element_count);
+    put<float>(out, t.scale);
+    put<float>(out, t.threshold);
+    put<uint64_t>(out, (uint64_t)t.packed_data.size());
+    for (size_t d : t.shape) put<uint64_t>(out, (uint64_t)d);
+    out.insert(out.end(), t.packed_data.begin(), t.packed_data.end());
+    put<uint32_t>(out, crc32_ieee(out.data(), out.size()));
+    FILE *f = std::fopen(path.c_str(), "wb");
+    if (!f) throw Error("cannot open " + path + " for writing");
+    const size_t w = std::fwrite(out.data(), 1, out.size(), f);
+    const int rc = std::fclose(f);
+    if (w != out.size() || rc != 0) throw Error("short write to " + path);
+}
+
+TernaryTensor load_ternary_tensor(const std::string &path) {
+    FILE *f = std::fopen(path.c_str(), "rb");
+    if (!f) throw Error("cannot open " + path);
+    std::vector<uint8_t> in;
+    uint8_t buf[1 << 16];
+    size_t r;
+    while ((r = std::fread(buf, 1, sizeof(buf), f)) > 0) in.insert(in.end(), buf, buf + r);
+    std::fclose(f);
+    if (in.size() < 44 || std::memcmp(in.data(), kMagic, 8) != 0)
+        throw Error(path + " is not a packed-weight file");
+    size_t off = 8;
+    const uint32_t version = get<uint32_t>(in, off), ndim = get<uint32_t>(in, off);
+    if (version != 1) throw Error("packed-weight file: unsupported version");
+    if (ndim > 8) throw Error("packed-weight file: more than 8 dimensions");
+    TernaryTensor t;
+    t.element_count = (size_t)get<uint64_t>(in, off);
+    t.scale = get<float>(in, off);
+    t.threshold = get<float>(in, off);
+    const uint64_t packed = get<uint64_t>(in, off);
+    for (uint32_t i = 0; i < ndim; ++i) t.shape.push_back((size_t)get<uint64_t>(in, off));
+    if (packed > in.size() || off + packed + 4 != in.size())
+        throw Error("packed-weight file: size does not match its header");
+    t.packed_data.assign(in.begin() + off, in.begin() + off + packed);
+    off += packed;
+    const uint32_t want = get<uint32_t>(in, off);
+    if (crc32_ieee(in.data(), in.size() - 4) != want) throw Error("packed-weight file: checksum mismatch");
+    validate_ternary_tensor(t);
+    return t;
 }
 
 std::vector<Tensor> BitNetKernel::execute(const std::vector<Tensor> &inputs) {

@@ -73,6 +73,19 @@ struct TernaryTensor {
     int8_t get_value(size_t index) const;
 };
 
+// Packed-weight file: ternarisation becomes a one-time offline step.  The reference has the
+// fields (quantization.rs:249-260) but no serialisation; the format is this build's:
+//   0  "RBNTERN1"            8 bytes
+//   8  u32 version (1)      12  u32 ndim (<= 8)
+//  16  u64 element_count    24  f32 scale     28  f32 threshold
+//  32  u64 packed_bytes (= ceil(element_count / 4))
+//  40  u64 shape[ndim]      then the packed bytes (reference layout), then
+//  u32 CRC-32 (IEEE) of everything before it.  Little-endian throughout.
+void save_ternary_tensor(const TernaryTensor &t, const std::string &path);
+TernaryTensor load_ternary_tensor(const std::string &path);
+// Checks the invariants that quantize_ternary guarantees (sizes, zero tail bits).
+void validate_ternary_tensor(const TernaryTensor &t);
+
 // quantization.rs:24-208 (ternary half)
 class BitNetQuantizer {
    public:
@@ -103,6 +116,9 @@ class BitNetKernel : public CompiledKernel {
                  bool cache_weights, size_t max_cache_bytes);
     ~BitNetKernel() override;
     std::vector<Tensor> execute(const std::vector<Tensor> &inputs) override;
+    // TernaryMatMul with weights that are already ternarised (e.g. loaded from a packed
+    // weight file): A [m,k] f32 is quantised as in execute(), B comes from `w` ([k,n]).
+    Tensor execute_prepacked(const Tensor &a, const TernaryTensor &w);
     MemoryUsage get_memory_usage() const override;
     KernelStats get_performance_stats() const override;
 
@@ -113,6 +129,12 @@ class BitNetKernel : public CompiledKernel {
         size_t bytes = 0;
     };
     Tensor execute_ternary_matmul(const Tensor &a, const Tensor &b);
+    // the shared tail: quantise A, multiply, download
+    Tensor multiply(const Tensor &a, size_t m, size_t k, size_t n, const void *d_tiled, float w_scale);
+    // tiled device copy of packed weights, cached by `key` when caching is on; *owned tells
+    // the caller to free it
+    CachedWeights tiled_weights(uint64_t key, size_t k, size_t n, const uint8_t *h_packed,
+                                const float *h_f32, float scale, bool *owned);
     void update_stats(double us);  // kernels.rs:235-251
 
     BitNetOperation operation_;

@@ -326,6 +326,67 @@ int rbp_ternary_packed(rbp_ternary *t, uint8_t *h_out, uint64_t capacity) {
     });
 }
 
+int rbp_ternary_from_parts(const uint8_t *h_packed, uint64_t packed_bytes, const uint64_t *shape,
+                           int ndim, float scale, float threshold, rbp_ternary **out) {
+    return guarded([&] {
+        if (!out || (!h_packed && packed_bytes) || (!shape && ndim > 0)) throw Error("null argument");
+        if (ndim < 0 || ndim > 8) throw Error("ndim must be in [0, 8]");
+        auto t = std::make_unique<rbp_ternary>();
+        t->t.packed_data.assign(h_packed, h_packed + packed_bytes);
+        size_t n = 1;
+        for (int i = 0; i < ndim; ++i) {
+            t->t.shape.push_back((size_t)shape[i]);
+            n *= (size_t)shape[i];
+        }
+        t->t.element_count = n;
+        t->t.scale = scale;
+        t->t.threshold = threshold;
+        validate_ternary_tensor(t->t);
+        *out = t.release();
+    });
+}
+
+int rbp_ternary_shape(rbp_ternary *t, uint64_t shape[8], int *ndim) {
+    return guarded([&] {
+        if (!t || !shape || !ndim) throw Error("null argument");
+        *ndim = (int)t->t.shape.size();
+        for (size_t i = 0; i < t->t.shape.size() && i < 8; ++i) shape[i] = t->t.shape[i];
+    });
+}
+
+int rbp_ternary_save(rbp_ternary *t, const char *path) {
+    return guarded([&] {
+        if (!t || !path) throw Error("null argument");
+        save_ternary_tensor(t->t, path);
+    });
+}
+
+int rbp_ternary_load(const char *path, rbp_ternary **out) {
+    return guarded([&] {
+        if (!path || !out) throw Error("null argument");
+        auto t = std::make_unique<rbp_ternary>();
+        t->t = load_ternary_tensor(path);
+        *out = t.release();
+    });
+}
+
+int rbp_kernel_execute_prepacked(rbp_kernel *k, const float *h_a, const uint64_t *shape_a, int ndim_a,
+                                 rbp_ternary *w, float *h_out, uint64_t out_capacity,
+                                 uint64_t out_shape[2]) {
+    return guarded([&] {
+        if (!k || !w || !h_out) throw Error("null argument");
+        auto *bk = dynamic_cast<BitNetKernel *>(k->k.get());
+        if (!bk) throw Error("not a BitNet kernel");
+        Tensor r = bk->execute_prepacked(make_tensor(h_a, shape_a, ndim_a, 0), w->t);
+        if (r.numel() > out_capacity) throw Error("output buffer too small");
+        std::copy(r.to_vec().begin(), r.to_vec().end(), h_out);
+        if (out_shape) {
+            out_shape[0] = r.shape()[0];
+            out_shape[1] = r.shape()[1];
+        }
+    });
+}
+
 int rbp_ternary_get_value(rbp_ternary *t, uint64_t index) {
     return t ? (int)t->t.get_value((size_t)index) : 0;
 }

@@ -265,3 +265,22 @@ def test_allocator(provider):                                     # allocator.rs
     alloc.deallocate(f)
     with pytest.raises(Error, match="Unsupported data type for BitNet allocator"):
         alloc.allocate([4], DataType.I32)
+
+
+def test_execute_with_weights_from_a_packed_file(provider, tmp_path):
+    """Ternarise once, save, load, execute: same bits as execute() on the f32 weights."""
+    from ronn_amd.bitnet import BitNetQuantizer, TernaryTensor
+    a = synth_normal(71, 1.0, (5, 300))
+    w = synth_normal(72, 0.02, (300, 77))
+    tw = BitNetQuantizer(QuantizationMethod.Ternary, provider).quantize_ternary(Tensor.from_data(w, [300, 77]))
+    path = tmp_path / "layer.rbnt"
+    tw.save(path)
+    loaded = TernaryTensor.load(path)
+    assert loaded.shape == [300, 77] and (loaded.packed_data == tw.packed_data).all()
+    kernel = provider.create_ternary_matmul_kernel(0, 0, 0)
+    want = kernel.execute([Tensor.from_data(a, [5, 300]), Tensor.from_data(w, [300, 77])])[0].numpy()
+    got = kernel.execute_prepacked(Tensor.from_data(a, [5, 300]), loaded).numpy()
+    assert got.shape == (5, 77) and same_bits(got, want)
+    assert kernel.get_performance_stats().execution_count == 2
+    with pytest.raises(Error, match="Matrix dimension mismatch"):
+        kernel.execute_prepacked(Tensor.from_data(a[:, :299].copy(), [5, 299]), loaded)

@@ -163,3 +163,54 @@ def test_blas_helper_equals_literal_oracle_loop():
         acc2 = exact_int_matmul(q, t.values().reshape(k, n))
         assert (acc == acc2).all()
         assert (out.view(np.uint32) == epilogue(acc2, s, t.scale).view(np.uint32)).all()
+
+
+# ---- packed-weight files (no GPU needed) ----------------------------------------------------------
+
+def test_packed_weight_file_round_trip(lib, tmp_path):
+    from ronn_amd import bitnet
+    rng = np.random.default_rng(9)
+    for shape in ((64, 64), (7, 13), (5,), (2, 3, 4), (1, 1)):
+        w = rng.normal(0, 0.02, shape).astype(np.float32)
+        t = O.quantize_ternary(w)
+        tt = bitnet.TernaryTensor.from_parts(t.packed_data, list(shape), t.scale, t.threshold)
+        path = tmp_path / ("w_%s.rbnt" % "x".join(map(str, shape)))
+        tt.save(path)
+        back = bitnet.TernaryTensor.load(path)
+        assert back.shape == list(shape) and back.element_count == w.size
+        assert (back.packed_data == t.packed_data).all()
+        assert np.float32(back.scale).view(np.uint32) == np.float32(t.scale).view(np.uint32)
+        assert np.float32(back.threshold).view(np.uint32) == np.float32(t.threshold).view(np.uint32)
+        assert [back.get_value(i) for i in range(min(w.size, 50))] == list(t.values()[:50])
+        raw = open(path, "rb").read()
+        assert raw[:8] == b"RBNTERN1" and len(raw) == 40 + 8 * len(shape) + (w.size + 3) // 4 + 4
+
+
+def test_packed_weight_file_rejects_damage(lib, tmp_path):
+    from ronn_amd import bitnet
+    w = np.random.default_rng(10).normal(0, 0.02, (16, 9)).astype(np.float32)
+    t = O.quantize_ternary(w)
+    good = tmp_path / "good.rbnt"
+    bitnet.TernaryTensor.from_parts(t.packed_data, [16, 9], t.scale, t.threshold).save(good)
+    raw = bytearray(open(good, "rb").read())
+    cases = {"flipped payload bit": (60, raw[60] ^ 4), "bad magic": (0, ord("X")), "version": (8, 2)}
+    for name, (off, val) in cases.items():
+        bad = bytearray(raw)
+        bad[off] = val
+        p = tmp_path / "bad.rbnt"
+        open(p, "wb").write(bad)
+        with pytest.raises(bitnet.Error):
+            bitnet.TernaryTensor.load(p)
+    open(tmp_path / "short.rbnt", "wb").write(raw[:-7])
+    with pytest.raises(bitnet.Error, match="size|truncated"):
+        bitnet.TernaryTensor.load(tmp_path / "short.rbnt")
+    with pytest.raises(bitnet.Error, match="cannot open"):
+        bitnet.TernaryTensor.load(tmp_path / "missing.rbnt")
+    # from_parts enforces the quantiser's invariants
+    with pytest.raises(bitnet.Error, match="packed size"):
+        bitnet.TernaryTensor.from_parts(t.packed_data[:-1], [16, 9], 1.0, 0.0)
+    odd = O.quantize_ternary(np.ones(5, np.float32))
+    dirty = odd.packed_data.copy()
+    dirty[-1] |= 0x80
+    with pytest.raises(bitnet.Error, match="tail bits"):
+        bitnet.TernaryTensor.from_parts(dirty, [5], 1.0, 0.0)

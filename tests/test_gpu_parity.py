@@ -404,3 +404,37 @@ def test_mfma_probe_reports_a_plausible_rate(ctx):
     assert 1000 < tern <= const * 1.05 < 5500
     with pytest.raises(_lib.RbnError):
         ctx.probe_mfma_i8(7)
+
+
+def test_captured_graph_replays_match_eager_results(ctx):
+    """A graph of matmuls (GEMV, small-batch kernel with its cross-workgroup k split and
+    ticket counters, MFMA GEMM) replayed several times, with eager work in between, gives
+    the eager bits on every replay."""
+    cases = []
+    for M, K, N in ((1, 2048, 2048), (8, 4096, 1024), (16, 11008, 512), (200, 512, 384)):
+        x = synth_normal(0x5EED0008 + M, 1.0, (M, K))
+        w = synth_normal(0x5EED1008 + N, 0.02, (K, N))
+        d_w = ctx.to_device(w)
+        d_p, w_scale, _, _ = ctx.quantize_ternary(d_w, w.size)
+        d_t = ctx.tile_weights(d_p, K, N)
+        acts = ctx.act_quant_i8(ctx.to_device(x), M, K)
+        eager, _ = ctx.matmul(acts, d_t, w_scale, M, K, N)
+        cases.append((M, K, N, acts, d_t, w_scale, eager.download(np.float32, M * N), ctx.alloc(4 * M * N)))
+    ctx.sync()
+    ctx.graph_begin()
+    for M, K, N, acts, d_t, w_scale, _, d_out in cases:
+        ctx.matmul(acts, d_t, w_scale, M, K, N, d_out=d_out)
+    g = ctx.graph_end()
+    for rep in range(4):
+        for c in cases:
+            check_fill = ctx.lib.rbn_fill_u8(ctx.handle, c[7].ptr, 0xFF, 4 * c[0] * c[2])
+            assert check_fill == 0
+        ctx.graph_launch(g)
+        ctx.sync()
+        for M, K, N, acts, d_t, w_scale, want, d_out in cases:
+            assert same_bits(d_out.download(np.float32, M * N), want), (rep, M, K, N)
+        # eager work between replays (uses the same workspace and ticket counters)
+        M, K, N, acts, d_t, w_scale, want, _ = cases[rep % len(cases)]
+        again, _ = ctx.matmul(acts, d_t, w_scale, M, K, N)
+        assert same_bits(again.download(np.float32, M * N), want)
+    ctx.graph_destroy(g)

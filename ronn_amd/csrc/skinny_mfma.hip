@@ -69,19 +69,21 @@ __device__ __forceinline__ v4i as_v4i(uint4 a) {
     return r;
 }
 
-// MT row tiles of 16 tokens, D steps of loads in flight, REFILL: some wave's range is longer
-// than D steps, MAXW: most waves per workgroup (sets the register budget).
-template <int MT, int D, bool REFILL, int MAXW>
+// MT row tiles of 16 tokens, NG groups of 64 columns per wave (the activation fragments are
+// loaded once and used for all of them: with four row tiles the activations, not the
+// weights, are most of the traffic), D steps of loads in flight, REFILL: some wave's range
+// is longer than D steps, MAXW: most waves per workgroup (sets the register budget).
+template <int MT, int NG, int D, bool REFILL, int MAXW>
 __global__ __launch_bounds__(MAXW * 64) void skinny_t2_i8_kernel(
     const int8_t *__restrict__ q,         // [M][Kpad], Kpad % 128 == 0
     const float *__restrict__ act_scale,  // [M]
     const int32_t *__restrict__ rowsum,   // [M]
     const uint4 *__restrict__ wt,         // tiled: uint4 index quad * KB + kb
     float w_scale, int M, int Kpad, int N, int groups, int splits,
-    int4 *__restrict__ partials,      // [groups][splits][MT * 16 rows][16 quads], splits > 1
+    int4 *__restrict__ partials,      // [groups][splits][MT * 16 rows][NG * 16 quads], splits > 1
     unsigned *__restrict__ tickets,   // [groups], zero between launches
     int32_t *__restrict__ acc_out, float *__restrict__ out) {
-    extern __shared__ int4 red[];  // [waves][MT * 16 rows][16 quads]
+    extern __shared__ int4 red[];  // [waves][MT * 16 rows][NG * 16 quads]
     __shared__ int s_last;
 
     const int tid = threadIdx.x;
@@ -98,38 +100,49 @@ __global__ __launch_bounds__(MAXW * 64) void skinny_t2_i8_kernel(
     const int s0 = gw * steps / gn, s1 = (gw + 1) * steps / gn;
 
     // a step advances both operands by four 16-byte units
-    const uint4 *wp = wt + (size_t)(group * 16 + ql) * KB + g;
+    const int cgroups = (int)(((size_t)N + 63) >> 6);  // groups of 64 columns that exist
+    const uint4 *wp[NG];
+#pragma unroll
+    for (int ng = 0; ng < NG; ++ng)
+        wp[ng] = wt + (size_t)(min(group * NG + ng, cgroups - 1) * 16 + ql) * KB + g;
     const uint4 *ap[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
         ap[mt] = reinterpret_cast<const uint4 *>(q + (size_t)min(mt * 16 + ql, M - 1) * Kpad) + g;
 
-    v4i acc[MT][4];
+    v4i acc[NG][MT][4];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int ng = 0; ng < NG; ++ng)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[mt][j] = v4i{0, 0, 0, 0};
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[ng][mt][j] = v4i{0, 0, 0, 0};
 
-    uint4 wr[D], ar[D][MT];
+    uint4 wr[D][NG], ar[D][MT];
 #pragma unroll
     for (int d = 0; d < D; ++d) {
         const int s = min(s0 + d, s1 - 1);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) ar[d][mt] = ap[mt][4 * s];
-        wr[d] = wp[4 * s];
+#pragma unroll
+        for (int ng = 0; ng < NG; ++ng) wr[d][ng] = wp[ng][4 * s];
         // same issue order as the reloads in the loop, so that one wait count fits both
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    auto consume = [&](const uint4 &w, const uint4 (&a)[MT]) {
-        const v4i b0 = decode_b(w.x), b1 = decode_b(w.y), b2 = decode_b(w.z), b3 = decode_b(w.w);
+    auto consume = [&](const uint4 (&w)[NG], const uint4 (&a)[MT]) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const v4i af = as_v4i(a[mt]);
-            acc[mt][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, b0, acc[mt][0], 0, 0, 0);
-            acc[mt][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, b1, acc[mt][1], 0, 0, 0);
-            acc[mt][2] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, b2, acc[mt][2], 0, 0, 0);
-            acc[mt][3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, b3, acc[mt][3], 0, 0, 0);
+        for (int ng = 0; ng < NG; ++ng) {
+            const v4i b0 = decode_b(w[ng].x), b1 = decode_b(w[ng].y), b2 = decode_b(w[ng].z),
+                      b3 = decode_b(w[ng].w);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const v4i af = as_v4i(a[mt]);
+                acc[ng][mt][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, b0, acc[ng][mt][0], 0, 0, 0);
+                acc[ng][mt][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, b1, acc[ng][mt][1], 0, 0, 0);
+                acc[ng][mt][2] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, b2, acc[ng][mt][2], 0, 0, 0);
+                acc[ng][mt][3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, b3, acc[ng][mt][3], 0, 0, 0);
+            }
         }
     };
 
@@ -157,28 +170,31 @@ __global__ __launch_bounds__(MAXW * 64) void skinny_t2_i8_kernel(
                 const int sn = min(base + d + D, s1 - 1);
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) ar[d][mt] = ap[mt][4 * sn];
-                wr[d] = wp[4 * sn];
+#pragma unroll
+                for (int ng = 0; ng < NG; ++ng) wr[d][ng] = wp[ng][4 * sn];
             }
             __builtin_amdgcn_sched_barrier(0);
         }
         base += D;
     } while (REFILL && base < s1);
 
-    // Meet through LDS.  acc[mt][j][i] is row mt*16 + 4*g + i, column 4*ql + j of the
-    // workgroup's 64 columns: one int4 per (row, quad).
-    const int rows = MT * 16;
+    // Meet through LDS.  acc[ng][mt][j][i] is row mt*16 + 4*g + i, column 4*ql + j of the
+    // ng-th group of 64 columns: one int4 per (row, quad).
+    constexpr int rows = MT * 16, quads = NG * 16;
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int ng = 0; ng < NG; ++ng)
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            red[(wave * rows + mt * 16 + 4 * g + i) * 16 + ql] =
-                make_int4(acc[mt][0][i], acc[mt][1][i], acc[mt][2][i], acc[mt][3][i]);
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                red[(wave * rows + mt * 16 + 4 * g + i) * quads + ng * 16 + ql] = make_int4(
+                    acc[ng][mt][0][i], acc[ng][mt][1][i], acc[ng][mt][2][i], acc[ng][mt][3][i]);
     __syncthreads();
 
     const bool vec_ok = (N & 3) == 0;
     auto finish = [&](int idx, int4 t) {
-        const int row = idx >> 4, qd = idx & 15;
-        const int col0 = (group * 16 + qd) * 4;
+        const int row = idx / quads, qd = idx - row * quads;
+        const int col0 = (group * quads + qd) * 4;
         if (row >= M || col0 >= N) return;
         const int rs = rowsum[row];
         const float as = act_scale[row];
@@ -204,7 +220,7 @@ __global__ __launch_bounds__(MAXW * 64) void skinny_t2_i8_kernel(
         }
     };
 
-    const int tile = rows * 16;  // int4 entries of one partial tile
+    constexpr int tile = rows * quads;  // int4 entries of one partial tile
     int4 *mine = partials + ((size_t)group * splits + split) * tile;
     for (int idx = tid; idx < tile; idx += blockDim.x) {
         int4 t = red[idx];
@@ -265,14 +281,14 @@ struct Args {
 };
 
 // Most waves per workgroup: bounded by registers (launch bounds) and by the reduction
-// buffer, waves * MT * 4 KiB of LDS.
-template <int MT>
-constexpr int max_waves() { return MT == 4 ? 8 : 16; }
+// buffer, waves * MT * NG * 4 KiB of LDS (at most 128 KiB).
+template <int MT, int NG>
+constexpr int max_waves() { return MT * NG >= 8 ? 4 : (MT * NG >= 4 ? 8 : 16); }
 
-template <int MT, int D, bool REFILL>
+template <int MT, int NG, int D, bool REFILL>
 int launch(hipStream_t stream, const Args &a) {
-    const size_t lds = (size_t)a.waves * MT * 16 * 16 * sizeof(int4);
-    auto kernel = skinny_t2_i8_kernel<MT, D, REFILL, max_waves<MT>()>;
+    const size_t lds = (size_t)a.waves * MT * NG * 16 * 16 * sizeof(int4);
+    auto kernel = skinny_t2_i8_kernel<MT, NG, D, REFILL, max_waves<MT, NG>()>;
     // more than the default 64 KiB of LDS has to be asked for, once per instantiation
     static const hipError_t attr = hipFuncSetAttribute(
         reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
@@ -284,17 +300,21 @@ int launch(hipStream_t stream, const Args &a) {
 }
 
 // D: the smallest ring that holds a wave's whole range, else the deepest with reloads.
-template <int MT>
+template <int MT, int NG>
 int launch_d(hipStream_t stream, const Args &a) {
     const int steps = a.Kpad / 64, gn = a.splits * a.waves;
     const int longest = (steps + gn - 1) / gn;  // a wave gets floor or ceil of steps / gn
-    if (longest <= 2) return launch<MT, 2, false>(stream, a);
-    if (longest <= 4) return launch<MT, 4, false>(stream, a);
-    if constexpr (MT == 1) {
-        if (longest <= 8) return launch<MT, 8, false>(stream, a);
-        return launch<MT, 8, true>(stream, a);
+    if (longest <= 2) return launch<MT, NG, 2, false>(stream, a);
+    if constexpr (MT * NG >= 8) {
+        return launch<MT, NG, 2, true>(stream, a);
     } else {
-        return launch<MT, 4, true>(stream, a);
+        if (longest <= 4) return launch<MT, NG, 4, false>(stream, a);
+        if constexpr (MT == 1) {
+            if (longest <= 8) return launch<MT, NG, 8, false>(stream, a);
+            return launch<MT, NG, 8, true>(stream, a);
+        } else {
+            return launch<MT, NG, 4, true>(stream, a);
+        }
     }
 }
 
@@ -324,25 +344,32 @@ extern "C" int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const floa
     a.M = (int)M;
     a.Kpad = (int)rbn_kpad(K);
     a.N = (int)N;
-    a.groups = (int)(rbn_npad(N) / 64);
     a.partials = (int4 *)ctx->splitk_partials;
     a.tickets = ctx->splitk_tickets;
     a.acc = d_acc;
     a.out = d_out;
     const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+    // four row tiles and a wide matrix: a wave takes two groups of 64 columns, which halves
+    // the activation traffic (8192 x 28672, M = 64: 55 -> 43 us); narrower matrices need
+    // the workgroups more than the saving (4096 x 11008: 18 us with one group, 28 with two)
+    const int cgroups = (int)(rbn_npad(N) / 64);
+    const int ng = (mt == 4 && cgroups >= 256) ? 2 : 1;
+    a.groups = (cgroups + ng - 1) / ng;
     // Shape of the launch (measured on the decode shapes; 64-k steps per wave in brackets).
-    // With 128 column groups or more, one workgroup per group: 4096 x 11008 runs 16 waves
-    // [4], 8192 x 28672 16 waves [8].  Narrower matrices are also split along k across
+    // With enough column groups, one workgroup per group: 4096 x 11008 runs 16 waves [4],
+    // 8192 x 28672 16 waves [8].  Narrower matrices are also split along k across
     // workgroups, towards ~256 of them; the round trip of the partial tiles through
     // memory costs 1-2 us, which is why wide matrices are not split.  A wave should get 4
     // steps (a ring of 4 with nothing masked), or 8 and more when the workgroup is full.
     const int steps = a.Kpad / 64;
-    const int max_w = mt == 4 ? max_waves<4>() : max_waves<1>();
+    const int max_w = mt == 4 ? (ng == 2 ? max_waves<4, 2>() : max_waves<4, 1>())
+                              : (mt == 2 ? max_waves<2, 1>() : max_waves<1, 1>());
     int splits = 1;
-    if (a.groups < 128) splits = (256 + a.groups - 1) / a.groups;
+    if (a.groups < 128 || a.groups * max_w < 1024) splits = (256 + a.groups - 1) / a.groups;
     if (splits > steps / 4) splits = steps / 4 > 0 ? steps / 4 : 1;
     // the workspace holds RBN_SPLITK_TILES tiles of 16 x 64 int32 and one ticket per group
-    while (splits > 1 && ((int64_t)a.groups * splits * mt > RBN_SPLITK_TILES || a.groups > RBN_SPLITK_GROUPS))
+    while (splits > 1 &&
+           ((int64_t)a.groups * splits * mt * ng > RBN_SPLITK_TILES || a.groups > RBN_SPLITK_GROUPS))
         --splits;
     const int steps_per_split = (steps + splits - 1) / splits;
     int waves = (steps_per_split + 3) / 4;
@@ -353,9 +380,9 @@ extern "C" int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const floa
     a.waves = waves;
     int rc;
     switch (mt) {
-        case 1: rc = launch_d<1>(ctx->stream, a); break;
-        case 2: rc = launch_d<2>(ctx->stream, a); break;
-        default: rc = launch_d<4>(ctx->stream, a); break;
+        case 1: rc = launch_d<1, 1>(ctx->stream, a); break;
+        case 2: rc = launch_d<2, 1>(ctx->stream, a); break;
+        default: rc = ng == 2 ? launch_d<4, 2>(ctx->stream, a) : launch_d<4, 1>(ctx->stream, a); break;
     }
     RBN_CHECK(rc);
     RBN_HIP(hipGetLastError());

@@ -332,6 +332,16 @@ def test_skinny_sweep_shapes(ctx, M, K, N):
     check_against_oracle(x, w, *res, literal=False)
 
 
+@pytest.mark.parametrize("M,K,N", [(64, 256, 16400), (33, 192, 16384), (50, 128, 20000)])
+def test_skinny_two_column_groups_per_wave(ctx, M, K, N):
+    # wide matrices with four row tiles take two groups of 64 columns per wave; odd group
+    # counts and ragged N exercise the clamped last group
+    x = synth_normal(0x5EED0009 + M, 1.0, (M, K))
+    w = synth_normal(0x5EED1009 + N, 0.02, (K, N))
+    res = run_matmul(ctx, ctx.skinny, x, w)
+    check_against_oracle(x, w, *res, literal=False)
+
+
 def test_skinny_saturated_activations(ctx):
     M, K, N = 48, 8192, 128
     x = np.where(synth_normal(7, 1.0, (M, K)) > 0, 1.0, -1.0).astype(np.float32)

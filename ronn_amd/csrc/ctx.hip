@@ -99,6 +99,11 @@ int rbn_ctx_create(int device, rbn_ctx **out) {
         rbn_ctx_destroy(ctx);
         return rc;
     }
+    const int prep = rbn_skinny_prepare();
+    if (prep != RBN_OK) {
+        rbn_ctx_destroy(ctx);
+        return prep;
+    }
     *out = ctx;
     return RBN_OK;
 }

@@ -288,15 +288,19 @@ constexpr int max_waves() { return MT * NG >= 8 ? 4 : (MT * NG >= 4 ? 8 : 16); }
 template <int MT, int NG, int D, bool REFILL>
 int launch(hipStream_t stream, const Args &a) {
     const size_t lds = (size_t)a.waves * MT * NG * 16 * 16 * sizeof(int4);
-    auto kernel = skinny_t2_i8_kernel<MT, NG, D, REFILL, max_waves<MT, NG>()>;
-    // more than the default 64 KiB of LDS has to be asked for, once per instantiation
-    static const hipError_t attr = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-    RBN_HIP(attr);
-    kernel<<<dim3((unsigned)(a.groups * a.splits)), dim3((unsigned)a.waves * 64), lds, stream>>>(
-        a.q, a.act_scale, a.rowsum, a.wt, a.w_scale, a.M, a.Kpad, a.N, a.groups, a.splits,
-        a.partials, a.tickets, a.acc, a.out);
+    skinny_t2_i8_kernel<MT, NG, D, REFILL, max_waves<MT, NG>()>
+        <<<dim3((unsigned)(a.groups * a.splits)), dim3((unsigned)a.waves * 64), lds, stream>>>(
+            a.q, a.act_scale, a.rowsum, a.wt, a.w_scale, a.M, a.Kpad, a.N, a.groups, a.splits,
+            a.partials, a.tickets, a.acc, a.out);
     return RBN_OK;
+}
+
+// More than the default 64 KiB of dynamic LDS has to be asked for per kernel function.
+template <int MT, int NG, int D, bool REFILL>
+hipError_t allow_large_lds() {
+    return hipFuncSetAttribute(
+        reinterpret_cast<const void *>(skinny_t2_i8_kernel<MT, NG, D, REFILL, max_waves<MT, NG>()>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
 }
 
 // D: the smallest ring that holds a wave's whole range, else the deepest with reloads.
@@ -319,6 +323,24 @@ int launch_d(hipStream_t stream, const Args &a) {
 }
 
 }  // namespace
+
+// Called once per context, outside any stream capture, for every instantiation that
+// launch_d can pick.
+int rbn_skinny_prepare() {
+    const hipError_t results[] = {
+        allow_large_lds<1, 1, 2, false>(), allow_large_lds<1, 1, 4, false>(),
+        allow_large_lds<1, 1, 8, false>(), allow_large_lds<1, 1, 8, true>(),
+        allow_large_lds<2, 1, 2, false>(), allow_large_lds<2, 1, 4, false>(),
+        allow_large_lds<2, 1, 4, true>(),  allow_large_lds<4, 1, 2, false>(),
+        allow_large_lds<4, 1, 4, false>(), allow_large_lds<4, 1, 4, true>(),
+        allow_large_lds<4, 2, 2, false>(), allow_large_lds<4, 2, 2, true>(),
+    };
+    for (hipError_t e : results)
+        if (e != hipSuccess)
+            return rbn_fail(RBN_ERR_HIP, "hipFuncSetAttribute(max dynamic LDS) failed: %s",
+                            hipGetErrorString(e));
+    return RBN_OK;
+}
 
 extern "C" int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
                                      const int32_t *d_rowsum, const uint32_t *d_tiled,

@@ -103,6 +103,47 @@ SEQ_HD SeqMap seq_append(SeqMap m, uint32_t ax_bits, uint32_t es) {
     return m;
 }
 
+// 2^(150 - es) as a float: multiplying a term by it expresses the term in units of the
+// state's ulp.  Representable for 23 <= es <= 276.
+SEQ_HD float seq_ulp_scale(uint32_t es) {
+    uint32_t bits = (277u - es) << 23;
+    float f;
+    __builtin_memcpy(&f, &bits, 4);
+    return f;
+}
+
+// seq_append for a term given as a non-negative float, with `scale` = seq_ulp_scale(es).
+// For es >= 26 the split of the term into (q, remainder) is done in floating point, which
+// takes a third fewer operations than the integer version and gives the same (q, >, ==):
+//   v = a * scale is exact (a power of two times a 24-bit mantissa) unless it overflows
+//   (a is far above the binade: saturate, as the integer version does for any term whose
+//   exponent exceeds the state's) or falls below 2^-126 (then a is below half an ulp
+//   whatever the rounding of v does, and for es >= 26 every subnormal a is in this case);
+//   floor(v) and v - floor(v) are exact for v < 2^25.
+// v in [2^24, 2^25) is not saturated here but yields q >= 2^24, which takes any k >= 2^23
+// past the limit just the same; the exact value of a map beyond the limit is never used.
+SEQ_HD SeqMap seq_append_abs(SeqMap m, float a, uint32_t es, float scale) {
+    if (es < 26u) {
+        uint32_t bits;
+        __builtin_memcpy(&bits, &a, 4);
+        return seq_append(m, bits, es);
+    }
+    const float v = a * scale;
+    uint32_t q = SEQ_SAT, gt = 0u, eq = 0u;
+    if (v < 33554432.0f) {  // false for NaN as well
+        const float fl = __builtin_floorf(v);
+        const float fr = v - fl;
+        q = (uint32_t)fl;
+        gt = fr > 0.5f ? 1u : 0u;
+        eq = fr == 0.5f ? 1u : 0u;
+    }
+    uint32_t t0 = m.d0 + q;
+    uint32_t t1 = m.d1 + q;
+    m.d0 = seq_min_u32(t0 + gt + (eq & (t0 & 1u)), SEQ_SAT);
+    m.d1 = seq_min_u32(t1 + gt + (eq & ((t1 + 1u) & 1u)), SEQ_SAT);
+    return m;
+}
+
 // Map of "first a, then b".
 SEQ_HD SeqMap seq_compose(SeqMap a, SeqMap b) {
     SeqMap r;
@@ -115,5 +156,27 @@ SEQ_HD SeqMap seq_compose(SeqMap a, SeqMap b) {
 
 // Applies a map to a concrete k.
 SEQ_HD uint32_t seq_apply(SeqMap m, uint32_t k) { return k + ((k & 1u) ? m.d1 : m.d0); }
+
+// ---- host-side window policy -------------------------------------------------------------
+// The block maps of a window are valid for one binade, so a window should end where S is
+// expected to leave it.  `s_now` is the current sum, `rate` its recent growth per block
+// (<= 0: unknown).  Without a rate the window is half again what has been summed so far
+// (S of similar terms doubles when the position doubles); with one, the distance to the
+// binade's upper edge at that rate plus a margin.  When growth slows down (rounding eats
+// more of every term in a higher binade) the window just ends early and the next one
+// continues with a fresh rate; blocks past a crossing are the only wasted reads.
+#include <math.h>
+static inline uint64_t seq_next_window(uint64_t pos, uint64_t total_blocks, double s_now, double rate) {
+    uint64_t win = pos + pos / 2;
+    if (rate > 0.0 && s_now > 0.0 && isfinite(s_now)) {
+        int e = 0;
+        (void)frexp(s_now, &e);  // s_now = m * 2^e, m in [0.5, 1): the binade ends at 2^e
+        const double need = (ldexp(1.0, e) - s_now) / rate;
+        win = need < 1e15 ? (uint64_t)(need * 1.06) + 4u : total_blocks;
+    }
+    if (win < 64u) win = 64u;
+    if (win > total_blocks - pos) win = total_blocks - pos;
+    return win;
+}
 
 #endif  // RONN_SEQSUM_CORE_H

@@ -149,7 +149,7 @@ __global__ __launch_bounds__(kBlock) void abs_sum_tree_final_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// Strict mode: the three kernels of the exact sequential sum (see seqsum_core.h).
+// Strict mode: the kernels of the exact sequential sum (see seqsum_core.h).
 // ---------------------------------------------------------------------------
 struct SeqState {
     uint32_t s_bits;       // current sum S as f32 bits (S >= 0)
@@ -167,6 +167,7 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
     __shared__ SeqMap s_wave[kBlock / 64];
     uint64_t base = first + (uint64_t)blockIdx.x * kSeqTile + (uint64_t)threadIdx.x * 16;
     SeqMap m = seq_identity();
+    const float scale = seq_ulp_scale(es < 26u ? 26u : es);
     if (base + 16 <= n) {
         float4 v[4];
 #pragma unroll
@@ -178,7 +179,7 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
             for (int i = 0; i < 4; ++i) {
                 float a = fabsf(e[i]);
                 bool take = use_mask ? (a > thr) : true;
-                if (take) m = seq_append(m, __float_as_uint(a), es);
+                if (take) m = seq_append_abs(m, a, es, scale);
             }
         }
     } else {
@@ -187,7 +188,7 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
             if (idx < n) {
                 float a = fabsf(x[idx]);
                 bool take = use_mask ? (a > thr) : true;
-                if (take) m = seq_append(m, __float_as_uint(a), es);
+                if (take) m = seq_append_abs(m, a, es, scale);
             }
         }
     }
@@ -207,122 +208,43 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
     }
 }
 
-// Walks the block maps of a window from the true state and finds the first block
-// in which k reaches 2^24.  One workgroup of 1024 threads.
-__global__ __launch_bounds__(1024) void seq_scan_kernel(const SeqMap *__restrict__ maps,
-                                                        uint32_t nblocks,
-                                                        SeqState *__restrict__ state) {
+// One workgroup of 1024 threads ends a window.
+// (1) Scan: walks the block maps of the window from the true state and finds the first
+//     block in which k reaches 2^24.
+// (2) Replay: resolves that block.  Its 256 chunks of 16 elements are mapped (threads
+//     0..255, one chunk each) and scanned from the state entering the block; the one chunk
+//     in which k reaches 2^24 is replayed with ordinary f32 additions, which moves S into a
+//     new binade; the chunks after it are mapped again for that binade, and so on to the
+//     end of the block.  Early blocks cross several binades (S doubles every few elements
+//     at first), later ones at most one.
+// The new state goes to device memory (for the next window's kernels) and to the pinned
+// host mailbox (the host reads it after synchronising: it sizes the next window).
+__global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
+    const SeqMap *__restrict__ maps, const float *__restrict__ x, uint64_t first, uint64_t n,
+    uint32_t nblocks, int use_mask, float thr, SeqState *__restrict__ state,
+    SeqState *__restrict__ host_copy) {
     __shared__ SeqMap s_a[1024];
     __shared__ SeqMap s_b[1024];
     __shared__ unsigned s_first;
+    __shared__ uint32_t s_cross_block, s_cross_k;
+    __shared__ uint32_t s_bits_now;
     const uint32_t t = threadIdx.x;
     uint32_t es, k0;
     seq_state_split(state->s_bits, &es, &k0);
-    const uint32_t chunk = (nblocks + 1023u) / 1024u;
-    const uint32_t lo = t * chunk;
-    const uint32_t hi = lo + chunk < nblocks ? lo + chunk : nblocks;
-    SeqMap mine = seq_identity();
-    for (uint32_t b = lo; b < hi; ++b) mine = seq_compose(mine, maps[b]);
-    if (t == 0) s_first = 0xffffffffu;
-    s_a[t] = mine;
-    __syncthreads();
-    // inclusive Hillis-Steele scan of the per-thread maps (order preserved)
-    SeqMap *src = s_a, *dst = s_b;
-    for (uint32_t off = 1; off < 1024u; off <<= 1) {
-        SeqMap v = src[t];
-        if (t >= off) v = seq_compose(src[t - off], v);
-        dst[t] = v;
-        __syncthreads();
-        SeqMap *tmp = src;
-        src = dst;
-        dst = tmp;
-    }
-    SeqMap before = t == 0 ? seq_identity() : src[t - 1];
-    uint32_t k = seq_apply(before, k0);
-    uint32_t cand = 0xffffffffu, cand_k = 0;
-    if (k < SEQ_K_LIMIT) {
-        for (uint32_t b = lo; b < hi; ++b) {
-            uint32_t k2 = seq_apply(maps[b], k);
-            if (k2 >= SEQ_K_LIMIT) {
-                cand = b;
-                cand_k = k;
-                break;
-            }
-            k = k2;
-        }
-    }
-    if (cand != 0xffffffffu) atomicMin(&s_first, cand);
-    __syncthreads();
-    const uint32_t first = s_first;
-    if (first != 0xffffffffu) {
-        if (cand == first) {
-            state->cross_block = first;
-            state->k = cand_k;
-        }
-    } else if (hi == nblocks && lo < hi) {
-        // this thread owns the last block of the window: k is the state after it
-        state->cross_block = 0xffffffffu;
-        state->k = k;
-    }
-}
 
-// Resolves the crossing block.  Its 256 chunks of 16 elements are mapped (one thread
-// each) and scanned from the state entering the block; the one chunk in which k reaches
-// 2^24 is replayed with ordinary f32 additions, which moves S into a new binade; the
-// chunks after it are mapped again for that binade, and so on to the end of the block.
-// Early blocks cross several binades (S doubles every few elements at first), later
-// ones at most one.
-__global__ __launch_bounds__(kBlock) void seq_replay_kernel(const float *__restrict__ x,
-                                                            uint64_t first, uint64_t n,
-                                                            uint32_t nblocks, int use_mask,
-                                                            float thr,
-                                                            SeqState *__restrict__ state) {
-    __shared__ SeqMap s_a[kBlock];
-    __shared__ SeqMap s_b[kBlock];
-    __shared__ unsigned s_first;
-    __shared__ uint32_t s_bits_now;
-    uint32_t es, k_cur;
-    seq_state_split(state->s_bits, &es, &k_cur);
-    const uint32_t cb = state->cross_block;
-    const uint32_t t = threadIdx.x;
-    if (cb == 0xffffffffu) {
-        if (t == 0) {
-            state->s_bits = seq_state_join(es, state->k);
-            state->next_rel = nblocks;
-        }
-        return;
-    }
-    k_cur = state->k;
-    const uint64_t base = first + (uint64_t)cb * kSeqTile + (uint64_t)t * 16;
-    float a[16];
-    bool take[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const uint64_t idx = base + i;
-        float v = 0.0f;
-        bool tk = false;
-        if (idx < n) {
-            v = fabsf(x[idx]);
-            tk = use_mask ? (v > thr) : true;
-        }
-        // a skipped element adds +0.0, which leaves any S >= 0 (and NaN/Inf) unchanged
-        a[i] = tk ? v : 0.0f;
-        take[i] = tk;
-    }
-    uint32_t done = 0;  // chunks [0, done) are already folded into (es, k_cur)
-    uint32_t result_bits = 0;
-    for (int guard = 0; guard <= kBlock; ++guard) {
-        SeqMap m = seq_identity();
-        if (t >= done) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i)
-                if (take[i]) m = seq_append(m, __float_as_uint(a[i]), es);
-        }
+    // ---- (1) scan -----------------------------------------------------------------------
+    {
+        const uint32_t chunk = (nblocks + 1023u) / 1024u;
+        const uint32_t lo = t * chunk;
+        const uint32_t hi = lo + chunk < nblocks ? lo + chunk : nblocks;
+        SeqMap mine = seq_identity();
+        for (uint32_t b = lo; b < hi; ++b) mine = seq_compose(mine, maps[b]);
         if (t == 0) s_first = 0xffffffffu;
-        s_a[t] = m;
+        s_a[t] = mine;
         __syncthreads();
+        // inclusive Hillis-Steele scan of the per-thread maps (order preserved)
         SeqMap *src = s_a, *dst = s_b;
-        for (uint32_t off = 1; off < (uint32_t)kBlock; off <<= 1) {
+        for (uint32_t off = 1; off < 1024u; off <<= 1) {
             SeqMap v = src[t];
             if (t >= off) v = seq_compose(src[t - off], v);
             dst[t] = v;
@@ -331,10 +253,112 @@ __global__ __launch_bounds__(kBlock) void seq_replay_kernel(const float *__restr
             src = dst;
             dst = tmp;
         }
-        const SeqMap before = t == 0 ? seq_identity() : src[t - 1];
-        const uint32_t k = seq_apply(before, k_cur);
-        const bool crosses = t >= done && k < SEQ_K_LIMIT && seq_apply(m, k) >= SEQ_K_LIMIT;
-        if (crosses) atomicMin(&s_first, t);
+        SeqMap before = t == 0 ? seq_identity() : src[t - 1];
+        uint32_t k = seq_apply(before, k0);
+        uint32_t cand = 0xffffffffu, cand_k = 0;
+        if (k < SEQ_K_LIMIT) {
+            for (uint32_t b = lo; b < hi; ++b) {
+                uint32_t k2 = seq_apply(maps[b], k);
+                if (k2 >= SEQ_K_LIMIT) {
+                    cand = b;
+                    cand_k = k;
+                    break;
+                }
+                k = k2;
+            }
+        }
+        if (cand != 0xffffffffu) atomicMin(&s_first, cand);
+        __syncthreads();
+        const uint32_t first_cross = s_first;
+        if (first_cross != 0xffffffffu) {
+            if (cand == first_cross) {
+                s_cross_block = first_cross;
+                s_cross_k = cand_k;
+            }
+        } else if (hi == nblocks && lo < hi) {
+            // this thread owns the last block of the window: k is the state after it
+            s_cross_block = 0xffffffffu;
+            s_cross_k = k;
+        }
+        __syncthreads();
+    }
+    const uint32_t cb = s_cross_block;
+    uint32_t k_cur = s_cross_k;
+    if (cb == 0xffffffffu) {
+        if (t == 0) {
+            const uint32_t bits = seq_state_join(es, k_cur);
+            state->s_bits = bits;
+            state->next_rel = nblocks;
+            host_copy->s_bits = bits;
+            host_copy->next_rel = nblocks;
+        }
+        return;
+    }
+
+    // ---- (2) replay of block cb: threads 0..255 hold a chunk, everybody keeps the barriers
+    const bool holds = t < (uint32_t)kBlock;
+    const uint64_t base = first + (uint64_t)cb * kSeqTile + (uint64_t)t * 16;
+    float a[16];
+    bool take[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        a[i] = 0.0f;
+        take[i] = false;
+    }
+    if (holds) {
+        if (base + 16 <= n && (reinterpret_cast<uintptr_t>(x + base) & 15u) == 0) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float4 v = reinterpret_cast<const float4 *>(x + base)[j];
+                a[4 * j] = fabsf(v.x), a[4 * j + 1] = fabsf(v.y), a[4 * j + 2] = fabsf(v.z), a[4 * j + 3] = fabsf(v.w);
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) take[i] = use_mask ? (a[i] > thr) : true;
+        } else {
+            for (int i = 0; i < 16; ++i) {
+                const uint64_t idx = base + i;
+                if (idx < n) {
+                    a[i] = fabsf(x[idx]);
+                    take[i] = use_mask ? (a[i] > thr) : true;
+                }
+            }
+        }
+        // a skipped element adds +0.0, which leaves any S >= 0 (and NaN/Inf) unchanged
+#pragma unroll
+        for (int i = 0; i < 16; ++i) a[i] = take[i] ? a[i] : 0.0f;
+    }
+    uint32_t done = 0;  // chunks [0, done) are already folded into (es, k_cur)
+    uint32_t result_bits = 0;
+    for (int guard = 0; guard <= kBlock; ++guard) {
+        SeqMap m = seq_identity();
+        if (holds && t >= done) {
+            const float scale = seq_ulp_scale(es < 26u ? 26u : es);
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                if (take[i]) m = seq_append_abs(m, a[i], es, scale);
+        }
+        if (t == 0) s_first = 0xffffffffu;
+        if (holds) s_a[t] = m;
+        __syncthreads();
+        SeqMap *src = s_a, *dst = s_b;
+        for (uint32_t off = 1; off < (uint32_t)kBlock; off <<= 1) {
+            if (holds) {
+                SeqMap v = src[t];
+                if (t >= off) v = seq_compose(src[t - off], v);
+                dst[t] = v;
+            }
+            __syncthreads();
+            SeqMap *tmp = src;
+            src = dst;
+            dst = tmp;
+        }
+        uint32_t k = 0;
+        if (holds) {
+            const SeqMap before = t == 0 ? seq_identity() : src[t - 1];
+            k = seq_apply(before, k_cur);
+            const bool crosses = t >= done && k < SEQ_K_LIMIT && seq_apply(m, k) >= SEQ_K_LIMIT;
+            if (crosses) atomicMin(&s_first, t);
+        }
         const uint32_t k_end = seq_apply(src[kBlock - 1], k_cur);  // state after the block if no crossing
         __syncthreads();
         const uint32_t tstar = s_first;
@@ -354,7 +378,7 @@ __global__ __launch_bounds__(kBlock) void seq_replay_kernel(const float *__restr
         if (((result_bits >> 23) & 0xffu) == 0xffu) {
             // S is +Inf or NaN.  +Inf turns into NaN if a NaN follows inside this block.
             bool nan_after = false;
-            if (t >= done) {
+            if (holds && t >= done) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) nan_after |= (a[i] != a[i]);
             }
@@ -370,6 +394,8 @@ __global__ __launch_bounds__(kBlock) void seq_replay_kernel(const float *__restr
     if (t == 0) {
         state->s_bits = result_bits;
         state->next_rel = cb + 1;
+        host_copy->s_bits = result_bits;
+        host_copy->next_rel = cb + 1;
     }
 }
 
@@ -482,30 +508,32 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     memset(h_state, 0, sizeof(SeqState));
     RBN_HIP(hipMemcpyAsync(&scr->seq, h_state, sizeof(SeqState), hipMemcpyHostToDevice,
                            ctx->stream));
-    RBN_HIP(hipStreamSynchronize(ctx->stream));
     uint64_t pos = 0;  // in blocks of kSeqTile elements
     uint32_t s_bits = 0;
+    double rate = 0.0;  // growth of S per block over the last window
     while (pos < total_blocks) {
         if (!is_finite_bits(s_bits)) break;
         uint32_t es, k;
         seq_state_split(s_bits, &es, &k);
-        uint64_t win = pos + pos / 2;
-        if (win < 64) win = 64;
-        if (win > total_blocks - pos) win = total_blocks - pos;
+        float s_before;
+        memcpy(&s_before, &s_bits, 4);
+        const uint64_t win = seq_next_window(pos, total_blocks, (double)s_before, rate);
         const uint64_t first = pos * kSeqTile;
         seq_block_maps_kernel<<<dim3((unsigned)win), dim3(kBlock), 0, ctx->stream>>>(
             d_x, first, n, es, use_mask, thr, maps);
-        seq_scan_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(maps, (uint32_t)win, &scr->seq);
-        seq_replay_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(d_x, first, n, (uint32_t)win,
-                                                                     use_mask, thr, &scr->seq);
+        // ends the window; also writes the new state to the pinned mailbox
+        seq_scan_replay_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(
+            maps, d_x, first, n, (uint32_t)win, use_mask, thr, &scr->seq, h_state);
         RBN_HIP(hipGetLastError());
-        RBN_HIP(hipMemcpyAsync(h_state, &scr->seq, sizeof(SeqState), hipMemcpyDeviceToHost,
-                               ctx->stream));
         RBN_HIP(hipStreamSynchronize(ctx->stream));
         s_bits = h_state->s_bits;
-        if (h_state->next_rel == 0 || h_state->next_rel > win)
+        const uint32_t advanced = h_state->next_rel;
+        if (advanced == 0 || advanced > win)
             return rbn_fail(RBN_ERR_HIP, "sequential-sum scan made no progress (internal error)");
-        pos += h_state->next_rel;
+        float s_after;
+        memcpy(&s_after, &s_bits, 4);
+        rate = ((double)s_after - (double)s_before) / (double)advanced;
+        pos += advanced;
     }
     float s;
     memcpy(&s, &s_bits, 4);

@@ -1,5 +1,5 @@
 // Host replica of the device's exact sequential-sum driver (ronn_amd/csrc/ternarize.hip:
-// seq_block_maps_kernel, seq_scan_kernel, seq_replay_kernel, strict_abs_sum), built on
+// seq_block_maps_kernel, seq_scan_replay_kernel, strict_abs_sum), built on
 // the same arithmetic header.  It lets the CPU test-suite check the algorithm against
 // a literal `s = s + |x|` loop on any input, without a GPU.
 #include <cmath>
@@ -14,16 +14,13 @@ constexpr int kTile = 4096;
 
 SeqMap thread_map(const float *x, uint64_t base, uint64_t n, uint32_t es, int use_mask, float thr) {
     SeqMap m = seq_identity();
+    const float scale = seq_ulp_scale(es < 26u ? 26u : es);
     for (int i = 0; i < 16; ++i) {
         uint64_t idx = base + i;
         if (idx < n) {
             float a = std::fabs(x[idx]);
             bool take = use_mask ? (a > thr) : true;
-            if (take) {
-                uint32_t bits;
-                std::memcpy(&bits, &a, 4);
-                m = seq_append(m, bits, es);
-            }
+            if (take) m = seq_append_abs(m, a, es, scale);
         }
     }
     return m;
@@ -121,13 +118,14 @@ extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr
     const uint64_t total_blocks = (n + kTile - 1) / kTile;
     uint64_t pos = 0;  // in blocks
     uint32_t s_bits = 0;
+    double rate = 0.0;
     while (pos < total_blocks) {
         if (((s_bits >> 23) & 0xff) == 0xff) break;
         uint32_t es, k;
         seq_state_split(s_bits, &es, &k);
-        uint64_t win = pos + pos / 2;
-        if (win < 64) win = 64;
-        if (win > total_blocks - pos) win = total_blocks - pos;
+        float s_before;
+        std::memcpy(&s_before, &s_bits, 4);
+        const uint64_t win = seq_next_window(pos, total_blocks, (double)s_before, rate);
         const uint64_t first = pos * kTile;
         std::vector<SeqMap> maps(win);
         for (uint64_t b = 0; b < win; ++b) maps[b] = block_map(x, first + b * kTile, n, es, use_mask, thr);
@@ -200,6 +198,9 @@ extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr
             s_bits = result_bits;
             next_rel = sr.cross_block + 1;
         }
+        float s_after;
+        std::memcpy(&s_after, &s_bits, 4);
+        rate = ((double)s_after - (double)s_before) / (double)next_rel;
         pos += next_rel;
         ++iters;
     }
@@ -230,4 +231,48 @@ extern "C" float seqsum_literal(const float *x, uint64_t n, int use_mask, float 
         if (take) s = s + a;
     }
     return s;
+}
+
+// Compares the floating-point term split (seq_append_abs, es >= 26) with the integer one
+// (seq_append) on `count` pseudo-random (map, term, exponent) triples.  Returns the number
+// of disagreements: below the limit the maps must be identical; at or above it both must
+// be at or above it (the exact value is never used there).
+extern "C" uint64_t seqsum_compare_term_splits(uint64_t count, uint64_t seed) {
+    uint64_t bad = 0, x = seed * 0x9E3779B97F4A7C15ull + 1;
+    auto next = [&]() {
+        x ^= x << 13;
+        x ^= x >> 7;
+        x ^= x << 17;
+        return x;
+    };
+    for (uint64_t i = 0; i < count; ++i) {
+        const uint32_t es = 26u + (uint32_t)(next() % 229u);  // 26 .. 254
+        SeqMap m;
+        m.d0 = (uint32_t)(next() % 5u == 0 ? next() % (1u << 24) : next() % 64u);
+        m.d1 = m.d0 + (uint32_t)(next() % 2u);
+        // a term near the state's ulp, sometimes far off, sometimes special
+        uint32_t ex = es - 30u + (uint32_t)(next() % 40u);  // es-30 .. es+9
+        if (next() % 16u == 0) ex = (uint32_t)(next() % 256u);
+        if (ex > 255u) ex = 0u;
+        uint32_t frac = (uint32_t)(next() & 0x7fffffu);
+        switch (next() % 8u) {
+            case 0: frac = 0; break;
+            case 1: frac &= 0x7f0000u; break;          // short mantissas: ties happen
+            case 2: frac = 0x400000u; break;
+            default: break;
+        }
+        const uint32_t bits = (ex << 23) | frac;
+        float a;
+        std::memcpy(&a, &bits, 4);
+        const SeqMap want = seq_append(m, bits, es);
+        const SeqMap got = seq_append_abs(m, a, es, seq_ulp_scale(es));
+        const bool w_over = want.d0 >= SEQ_K_LIMIT / 2 || want.d1 >= SEQ_K_LIMIT / 2;
+        if (w_over) {
+            // any increment of 2^23 or more ends the binade for every k >= 2^23
+            if (got.d0 < SEQ_K_LIMIT / 2 || got.d1 < SEQ_K_LIMIT / 2) ++bad;
+        } else if (got.d0 != want.d0 || got.d1 != want.d1) {
+            ++bad;
+        }
+    }
+    return bad;
 }

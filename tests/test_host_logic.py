@@ -104,6 +104,8 @@ def seqsum(tmp_path_factory):
                               C.POINTER(C.c_uint64)]
     L.seqsum_literal.restype = C.c_float
     L.seqsum_literal.argtypes = [C.c_void_p, C.c_uint64, C.c_int, C.c_float]
+    L.seqsum_compare_term_splits.restype = C.c_uint64
+    L.seqsum_compare_term_splits.argtypes = [C.c_uint64, C.c_uint64]
     return L
 
 
@@ -142,6 +144,12 @@ def test_parallel_sequential_sum_is_bit_exact(seqsum, name, x):
         want = np.float32(seqsum.seqsum_literal(x.ctypes.data, x.size, mask, thr))
         assert got.view(np.uint32) == want.view(np.uint32) or (np.isnan(got) and np.isnan(want)), \
             "%s mask=%d: %r vs %r" % (name, mask, got, want)
+
+
+def test_float_and_integer_term_splits_agree(seqsum):
+    # seq_append_abs (float split, used for es >= 26) against seq_append (integer split)
+    assert seqsum.seqsum_compare_term_splits(3_000_000, 1) == 0
+    assert seqsum.seqsum_compare_term_splits(1_000_000, 2) == 0
 
 
 def test_sequential_sum_traffic_is_bounded(seqsum):

@@ -34,11 +34,13 @@
 //    formats (zero activations, zero-weight codes), rows and columns past the edge are
 //    clamped duplicates whose results are never stored.
 #include "common.hpp"
+#include <type_traits>
 
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 typedef void __attribute__((address_space(3))) * lds_ptr;
 typedef const void __attribute__((address_space(1))) * global_ptr;
 
@@ -62,10 +64,10 @@ __device__ __forceinline__ v4i decode_b(uint32_t w) {
 
 // One wave-wide 16-byte-per-lane load from global memory straight into LDS: lane i's
 // 16 bytes land at LDS byte address lds_wave_base + 16 * i (M0 carries the base).
-__device__ __forceinline__ void dma16(const void *src, uint32_t lds_wave_base) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off"
+__device__ __forceinline__ void dma16(const void *base, uint32_t lane_offset, uint32_t lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
-                 : "s"(lds_wave_base), "v"(src)
+                 : "s"(lds_wave_base), "v"(lane_offset), "s"(base)
                  : "memory", "m0");
 }
 
@@ -121,19 +123,22 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
     // (4j + w) * 64 + lane: row (or quad) (4j + w) * 8 + lane / 8, slot lane % 8, and the
     // slot holds segment (or k-block) slot ^ ((row >> 1) & 7) of that row.
     const int sub = lane >> 3;
-    const int8_t *a_src[4];
+    // a workgroup-uniform base (scalar registers) plus a 32-bit byte offset per lane
+    const int8_t *a_base = q + (size_t)m0 * Kpad;
+    uint32_t a_lane[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const int lrow = (4 * j + wave) * 8 + sub;
         const int seg = (lane & 7) ^ ((lrow >> 1) & 7);
-        a_src[j] = q + (size_t)min(m0 + lrow, M - 1) * Kpad + seg * 16;
+        a_lane[j] = (uint32_t)(min(m0 + lrow, M - 1) - m0) * (uint32_t)Kpad + seg * 16;
     }
-    const uint4 *b_src[2];
+    const uint4 *b_base = wt + (size_t)q0 * KB;
+    uint32_t b_lane[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int lquad = (4 * j + wave) * 8 + sub;
         const int kb = (lane & 7) ^ ((lquad >> 1) & 7);
-        b_src[j] = wt + (size_t)min(q0 + lquad, nquads - 1) * KB + kb;
+        b_lane[j] = ((uint32_t)(min(q0 + lquad, nquads - 1) - q0) * (uint32_t)KB + kb) * 16;
     }
     const int iters = Kpad / BK;
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr)smem;
@@ -141,11 +146,12 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
         const int kk = min(it, iters - 1);  // past the end: reload the last step, never read
         const uint32_t sb = lds0 + (uint32_t)(stage * kBUnits) * 16;
         const uint32_t sa = lds0 + (uint32_t)(3 * kBUnits + stage * kAUnits) * 16;
+        const int8_t *ab = a_base + (size_t)kk * BK;
+        const uint4 *bb = b_base + (size_t)kk * (BK / 16);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) dma16(a_src[j] + (size_t)kk * BK, sa + (4 * j + wave) * 1024);
+        for (int j = 0; j < 4; ++j) dma16(ab, a_lane[j], sa + (4 * j + wave) * 1024);
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-            dma16(b_src[j] + (size_t)kk * (BK / 16), sb + (4 * j + wave) * 1024);
+        for (int j = 0; j < 2; ++j) dma16(bb, b_lane[j], sb + (4 * j + wave) * 1024);
     };
 
     // fragment addresses (in 16-byte units, relative to a stage)
@@ -233,8 +239,11 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
     // are outstanding (stage nxt has landed) and until this wave's reads of `cur` have
     // returned, meet, and go on with the reads of nxt.  In the last step nxt holds no
     // new data; what is read from it is never used.
-    int cur = 0, nxt = 1, fill = 2;
-    for (int it = 0; it < iters; ++it) {
+    // The loop body is written out for the three positions of the ring, so every LDS
+    // address is a lane constant plus an immediate.
+    auto kstep = [&](auto cur_tag, int it) {
+        constexpr int cur = decltype(cur_tag)::value;
+        constexpr int nxt = (cur + 1) % 3, fill = (cur + 2) % 3;
         issue(it + 2, fill);
         __builtin_amdgcn_sched_barrier(0);
         substep(0, cur, 2, 1);
@@ -244,11 +253,15 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
         __builtin_amdgcn_sched_barrier(0);
         substep(2, nxt, 0, 3);
         substep(3, nxt, 1, 0);
-        const int t = cur;
-        cur = nxt;
-        nxt = fill;
-        fill = t;
+    };
+    int it = 0;
+    for (; it + 2 < iters; it += 3) {
+        kstep(std::integral_constant<int, 0>{}, it);
+        kstep(std::integral_constant<int, 1>{}, it + 1);
+        kstep(std::integral_constant<int, 2>{}, it + 2);
     }
+    if (it < iters) kstep(std::integral_constant<int, 0>{}, it);
+    if (it + 1 < iters) kstep(std::integral_constant<int, 1>{}, it + 1);
     __builtin_amdgcn_s_waitcnt(kWaitVm0);  // no load may still be writing LDS at exit
 
     // epilogue: lane owns columns 4*quad .. 4*quad+3 (tile j -> column 4*quad + j) and rows
@@ -274,8 +287,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
             }
             const size_t o = (size_t)row * N + col0;
             if (vec_ok) {
-                *reinterpret_cast<float4 *>(out + o) = make_float4(v[0], v[1], v[2], v[3]);
-                if (acc_out) *reinterpret_cast<int4 *>(acc_out + o) = make_int4(t[0], t[1], t[2], t[3]);
+                __builtin_nontemporal_store(v4f{v[0], v[1], v[2], v[3]}, reinterpret_cast<v4f *>(out + o));
+                if (acc_out) __builtin_nontemporal_store(v4i{t[0], t[1], t[2], t[3]}, reinterpret_cast<v4i *>(acc_out + o));
             } else {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {

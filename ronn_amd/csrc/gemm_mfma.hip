@@ -13,8 +13,10 @@
 //    two row tiles per XCD and therefore misses L2) is covered by two K steps.  The loads
 //    are issued from inline assembly, so the compiler neither tracks nor waits for them;
 //    the ring is synchronised by hand: s_waitcnt vmcnt(6) leaves exactly the newest
-//    stage's six loads in flight, then a bare s_barrier.
-//  * A lane of such a load picks its own global address but lands at LDS base + 16 * lane,
+//    stage's six loads in flight, then a bare s_barrier.  The ring's three positions are
+//    written out in the loop body, so LDS addresses are lane constants plus immediates.
+//  * A lane of such a load picks its own global address (a workgroup-uniform base in scalar
+//    registers plus a 32-bit lane offset) but lands at LDS base + 16 * lane,
 //    so the LDS images are linear arrays of 16-byte units with an XOR swizzle chosen so
 //    that (a) eight consecutive lanes fetch one 128-byte line of global memory and (b) the
 //    128-bit fragment reads of eight consecutive lanes hit distinct banks:
@@ -26,7 +28,8 @@
 //  * Weights stay 2-bit until they are in registers.  Lane l reads ONE 16-byte unit (quad
 //    l%32, k-half l/32) per 32 k and expands it with 28 VALU operations into the B
 //    fragments of FOUR MFMA tiles: tile j covers the columns 4*quad + j.  The same mapping
-//    lets the epilogue store four adjacent columns per lane as one 128-bit store.
+//    lets the epilogue store four adjacent columns per lane as one 128-bit store
+//    (nontemporal: the output is written once and not read by this kernel).
 //  * Workgroups are numbered so that the eight XCDs each own a band of rows: a band's
 //    activations stay in that XCD's L2 while the weights stream through.
 //  * Weights are stored as code = value + 1, so the per-token sum of q is subtracted in

@@ -306,6 +306,19 @@ def test_gemm_mfma_small(ctx, M, K, N):
     check_against_oracle(x, w, *res, literal=(M * K * N <= 1 << 23))
 
 
+@pytest.mark.parametrize("M,K,N", [(2000, 128, 11016), (1030, 256, 15000), (1100, 384, 15000),
+                                   (2048, 512, 11008)])
+def test_gemm_mfma_more_than_one_round(ctx, M, K, N):
+    # more tiles than the 512 workgroups that fit the chip at once, with and without the
+    # XCD-aware numbering (16 and 9 row tiles), ragged M and N; K steps 1 to 4 cover every
+    # exit position of the three-stage ring
+    say("gemm rounds", M, K, N)
+    x = synth_normal(0x5EED000A + M, 1.0, (M, K))
+    w = synth_normal(0x5EED100A + N, 0.02, (K, N))
+    res = run_matmul(ctx, ctx.gemm, x, w)
+    check_against_oracle(x, w, *res, literal=False)
+
+
 @pytest.mark.parametrize("M", [1, 2, 3, 7, 16, 17, 31, 32, 33, 48, 64])
 @pytest.mark.parametrize("K,N", [(64, 64), (128, 64), (2048, 2048), (100, 37), (4096, 96), (130, 1376),
                                  (1100, 130)])

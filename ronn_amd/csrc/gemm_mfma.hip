@@ -48,12 +48,10 @@ typedef void __attribute__((address_space(3))) * lds_ptr;
 typedef const void __attribute__((address_space(1))) * global_ptr;
 
 constexpr int kThreads = 256;
-constexpr int BM = 128, BN = 256, BK = 128;
-constexpr int kAUnits = BM * 8;        // 16-byte units of one activation stage (16 KiB)
+constexpr int BN = 256, BK = 128;
 constexpr int kBUnits = (BN / 4) * 8;  // of one weight stage (8 KiB)
 
 // s_waitcnt immediates (gfx9 encoding: vmcnt[3:0] | expcnt << 4 | lgkmcnt << 8 | vmcnt[5:4] << 14)
-constexpr int kWaitVm6Lgkm0 = 0x0076;  // vmcnt(6) and lgkmcnt(0)
 constexpr int kWaitVm0 = 0x0F70;       // vmcnt(0)
 
 __device__ __forceinline__ v4i decode_b(uint32_t w) {
@@ -74,7 +72,11 @@ __device__ __forceinline__ void dma16(const void *base, uint32_t lane_offset, ui
                  : "memory", "m0");
 }
 
-__global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
+// MT = 2: the regular tile of 128 rows (waves of 64 x 128).  MT = 1: tiles of 64 rows (waves
+// of 32 x 128, half the accumulators, three workgroups per CU) for products whose 128-row
+// tiling would leave most of the chip idle.
+template <int MT>
+__global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_kernel(
     const int8_t *__restrict__ q,         // [M][Kpad], Kpad % 128 == 0
     const float *__restrict__ act_scale,  // [M]
     const int32_t *__restrict__ rowsum,   // [M]
@@ -83,9 +85,13 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
     int32_t *__restrict__ acc_out, float *__restrict__ out) {
     // Ring of three stages in one array (units of 16 bytes): weights of stage s at
     // s * kBUnits, activations at 3 * kBUnits + s * kAUnits.
+    constexpr int TM = 64 * MT;                  // rows of the tile
+    constexpr int kAUnits = TM * 8;              // 16-byte units of one activation stage
+    constexpr int kLoads = 2 * MT + 2;           // LDS loads per wave and stage
+    constexpr int kWaitStage = 0x0070 | kLoads;  // s_waitcnt vmcnt(kLoads) lgkmcnt(0)
     __shared__ __attribute__((aligned(16))) uint4 smem[3 * (kAUnits + kBUnits)];
-    __shared__ float s_scale[BM];
-    __shared__ int s_rowsum[BM];
+    __shared__ float s_scale[TM];
+    __shared__ int s_rowsum[TM];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -105,18 +111,18 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
         bm = blockIdx.x % m_tiles;
         bn = blockIdx.x / m_tiles;
     }
-    const int m0 = bm * BM, n0 = bn * BN;
+    const int m0 = bm * TM, n0 = bn * BN;
     const int q0 = n0 >> 2;
 
-    if (tid < BM) {
+    if (tid < TM) {
         const int row = m0 + tid;
         s_scale[tid] = row < M ? act_scale[row] : 0.0f;
         s_rowsum[tid] = row < M ? rowsum[row] : 0;
     }
 
-    v16i acc[2][4];
+    v16i acc[MT][4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < MT; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -128,9 +134,9 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
     const int sub = lane >> 3;
     // a workgroup-uniform base (scalar registers) plus a 32-bit byte offset per lane
     const int8_t *a_base = q + (size_t)m0 * Kpad;
-    uint32_t a_lane[4];
+    uint32_t a_lane[2 * MT];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < 2 * MT; ++j) {
         const int lrow = (4 * j + wave) * 8 + sub;
         const int seg = (lane & 7) ^ ((lrow >> 1) & 7);
         a_lane[j] = (uint32_t)(min(m0 + lrow, M - 1) - m0) * (uint32_t)Kpad + seg * 16;
@@ -152,13 +158,13 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
         const int8_t *ab = a_base + (size_t)kk * BK;
         const uint4 *bb = b_base + (size_t)kk * (BK / 16);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) dma16(ab, a_lane[j], sa + (4 * j + wave) * 1024);
+        for (int j = 0; j < 2 * MT; ++j) dma16(ab, a_lane[j], sa + (4 * j + wave) * 1024);
 #pragma unroll
         for (int j = 0; j < 2; ++j) dma16(bb, b_lane[j], sb + (4 * j + wave) * 1024);
     };
 
     // fragment addresses (in 16-byte units, relative to a stage)
-    const int frow0 = wm * 64 + (lane & 31), khalf = lane >> 5;
+    const int frow0 = wm * (32 * MT) + (lane & 31), khalf = lane >> 5;
     const int fquad = wn * 32 + (lane & 31);
     auto a_unit = [&](int row, int seg) { return row * 8 + (seg ^ ((row >> 1) & 7)); };
     auto b_unit = [&](int kb) { return fquad * 8 + (kb ^ ((fquad >> 1) & 7)); };
@@ -192,7 +198,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
         const uint4 *sa = smem + 3 * kBUnits + stage * kAUnits;
         rb[ks] = sb[b_off[ks]];
         ra0[ks] = sa[a_off[ks]];
-        ra1[ks] = sa[a_off[ks] + 32 * 8];  // row + 32: same swizzle
+        if constexpr (MT == 2) ra1[ks] = sa[a_off[ks] + 32 * 8];  // row + 32: same swizzle
     };
     auto decode_next = [&](int ks) {
         bf_n[0] = decode_b(rb[ks].x);
@@ -209,14 +215,16 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j)
             acc[0][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af0, bf[j], acc[0][j], 0, 0, 0);
+        if constexpr (MT == 2) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            acc[1][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af1, bf[j], acc[1][j], 0, 0, 0);
+            for (int j = 0; j < 4; ++j)
+                acc[1][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af1, bf[j], acc[1][j], 0, 0, 0);
+        }
 #pragma unroll
-        for (int g = 0; g < 8; ++g) {
-            if (g < 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);             // MFMA
-            __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);             // VALU
+        for (int g = 0; g < 4 * MT; ++g) {
+            if (g < MT + 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // MFMA
+            __builtin_amdgcn_sched_group_barrier(0x002, 8 / MT, 0);             // VALU
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) bf[j] = bf_n[j];
@@ -227,7 +235,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
     // then fill the pipeline: raw fragments of sub-steps 0 and 1, weights of 0 decoded
     issue(0, 0);
     issue(1, 1);
-    __builtin_amdgcn_s_waitcnt(kWaitVm6Lgkm0);
+    __builtin_amdgcn_s_waitcnt(kWaitStage);
     __builtin_amdgcn_s_barrier();
     lds_reads(0, 0);
     lds_reads(0, 1);
@@ -238,7 +246,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
 
     // K step `it` on stage cur: start the loads of step it+2 into `fill` - the stage read
     // in step it-1, which every wave has left: all its reads were waited for before the
-    // barrier inside step it-1.  After sub-step 1, wait until only those newest six loads
+    // barrier inside step it-1.  After sub-step 1, wait until only those newest kLoads loads
     // are outstanding (stage nxt has landed) and until this wave's reads of `cur` have
     // returned, meet, and go on with the reads of nxt.  In the last step nxt holds no
     // new data; what is read from it is never used.
@@ -251,7 +259,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
         __builtin_amdgcn_sched_barrier(0);
         substep(0, cur, 2, 1);
         substep(1, cur, 3, 2);
-        __builtin_amdgcn_s_waitcnt(kWaitVm6Lgkm0);
+        __builtin_amdgcn_s_waitcnt(kWaitStage);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         substep(2, nxt, 0, 3);
@@ -272,10 +280,10 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_t2_i8_mfma_kernel(
     const int col0 = n0 + fquad * 4;
     const bool vec_ok = (N & 3) == 0;
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt) {
+    for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int lrow = wm * 64 + mt * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const int lrow = wm * (32 * MT) + mt * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
             const int row = m0 + lrow;
             if (row >= M || col0 >= N) continue;
             const int rs = s_rowsum[lrow];
@@ -323,12 +331,22 @@ extern "C" int rbn_gemm_t2_i8_mfma(rbn_ctx *ctx, const int8_t *d_q, const float 
     const int Kpad = (int)rbn_kpad(K);
     static_assert(BK == 128, "the K padding of the formats must equal the K step");
     const int nquads = (int)(rbn_npad(N) / 4);
-    const int m_tiles = (int)((M + BM - 1) / BM), n_tiles = (int)((N + BN - 1) / BN);
+    // 128-row tiles, two workgroups per CU; when those would fill at most half of the slots,
+    // 64-row tiles (twice as many workgroups, three per CU)
+    const int n_tiles = (int)((N + BN - 1) / BN);
+    const uint64_t slots = 2ull * (uint64_t)ctx->props.multiProcessorCount;
+    const bool low = ((M + 127) / 128) * (uint64_t)n_tiles * 2 <= slots;
+    const int m_tiles = (int)((M + (low ? 63 : 127)) / (low ? 64 : 128));
     const uint64_t tiles = (uint64_t)m_tiles * n_tiles;
     RBN_REQUIRE(tiles <= 0x7fffffffull, "too many tiles");
-    gemm_t2_i8_mfma_kernel<<<dim3((unsigned)tiles), dim3(kThreads), 0, ctx->stream>>>(
-        d_q, d_act_scale, d_rowsum, (const uint4 *)d_tiled, w_scale, (int)M, Kpad, (int)N, nquads,
-        m_tiles, n_tiles, d_acc, d_out);
+    if (low)
+        gemm_t2_i8_mfma_kernel<1><<<dim3((unsigned)tiles), dim3(kThreads), 0, ctx->stream>>>(
+            d_q, d_act_scale, d_rowsum, (const uint4 *)d_tiled, w_scale, (int)M, Kpad, (int)N,
+            nquads, m_tiles, n_tiles, d_acc, d_out);
+    else
+        gemm_t2_i8_mfma_kernel<2><<<dim3((unsigned)tiles), dim3(kThreads), 0, ctx->stream>>>(
+            d_q, d_act_scale, d_rowsum, (const uint4 *)d_tiled, w_scale, (int)M, Kpad, (int)N,
+            nquads, m_tiles, n_tiles, d_acc, d_out);
     RBN_HIP(hipGetLastError());
     return RBN_OK;
 }

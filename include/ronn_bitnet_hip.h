@@ -235,7 +235,7 @@ int rbn_embed_f32(rbn_ctx *ctx, const float *d_table, const int32_t *d_tokens, u
 /* Input row: x[m,:] (H values); or, when d_delta is given, x += delta, written back
  * (the residual stream); or, when d_gate_up [M, 2H] is given instead of d_x,
  * x = silu(gate) * up (SwiGLU on the way in; nothing is written back).  Then
- * y = (x * rsqrt(mean(x^2) + eps)) * gamma, quantised per token exactly as
+ * y = (x * gamma) * rsqrt(mean(x^2) + eps), quantised per token exactly as
  * rbn_act_quant_i8 does (same output format).  H <= 8192. */
 int rbn_rmsnorm_quant_i8(rbn_ctx *ctx, float *d_x, const float *d_delta, const float *d_gate_up,
                          const float *d_gamma, float eps, uint64_t M, uint64_t H, int8_t *d_q,

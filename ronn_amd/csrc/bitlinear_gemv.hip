@@ -2,7 +2,7 @@
 // absmax int8 quantisation, ternary GEMV, fused dequantisation, optional residual add.
 //
 //   v      = x                         or  silu(gate) * up
-//   y      = (v * rsqrt(mean(v^2) + eps)) * gamma
+//   y      = (v * gamma) * rsqrt(mean(v^2) + eps)
 //   g      = max(max|y|, 1e-5);  q = clamp(rne(y * (127/g)), -128, 127);  s = g / 127
 //   out[n] = [residual[n] +] ((float)(sum_k q[k] * w[k,n]) * s) * w_scale
 //
@@ -22,7 +22,7 @@ namespace {
 
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
-constexpr int kMaxBlocksPerThread = 2;  // K <= 16 * 256 * 2 = 8192
+constexpr int kMaxBlocksPerThread = 2;  // K <= 16 * 256 * 2 = 8192 (template NB: 1 up to 4096)
 
 template <int CTRL, int ROWMASK>
 __device__ __forceinline__ int dpp_add(int v) {
@@ -38,16 +38,28 @@ __device__ __forceinline__ int wave_total_lane63(int v) {
     v = dpp_add<0x143, 0xC>(v);  // row_bcast31
     return v;
 }
-__device__ __forceinline__ float wave_sum_f(float v) {
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+// The same walk for floats (a fixed order, so every workgroup gets the same bits) and for
+// the maximum of non-negative floats; lanes outside a step's row mask see 0.
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROWMASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_sum_lane63(float v) {
+    v += dpp_f<0xB1, 0xf>(v);
+    v += dpp_f<0x4E, 0xf>(v);
+    v += dpp_f<0x124, 0xf>(v);
+    v += dpp_f<0x128, 0xf>(v);
+    v += dpp_f<0x142, 0xA>(v);
+    v += dpp_f<0x143, 0xC>(v);
     return v;
 }
-__device__ __forceinline__ float wave_max_f(float v) {
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    return v;
-}
-__device__ __forceinline__ int wave_sum_i(int v) {
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+__device__ __forceinline__ float wave_max_lane63(float v) {  // v >= 0
+    v = fmaxf(v, dpp_f<0xB1, 0xf>(v));
+    v = fmaxf(v, dpp_f<0x4E, 0xf>(v));
+    v = fmaxf(v, dpp_f<0x124, 0xf>(v));
+    v = fmaxf(v, dpp_f<0x128, 0xf>(v));
+    v = fmaxf(v, dpp_f<0x142, 0xA>(v));
+    v = fmaxf(v, dpp_f<0x143, 0xC>(v));
     return v;
 }
 
@@ -62,8 +74,9 @@ __device__ __forceinline__ uint4 to_nibble_planes(uint4 a) {
     return p;
 }
 
-// KS waves per column quad, L weight loads in flight per lane and round, SWIGLU input.
-template <int KS, int L, bool SWIGLU>
+// KS waves per column quad, L weight loads in flight per lane and round, SWIGLU input,
+// NB blocks of 16 activations per thread (K <= 4096 * NB).
+template <int KS, int L, bool SWIGLU, int NB>
 __global__ __launch_bounds__(kThreads) void bitlinear_gemv_kernel(
     const float *__restrict__ x,        // [K], or gate|up [2K] with SWIGLU
     const float *__restrict__ gamma,    // [K]
@@ -71,7 +84,7 @@ __global__ __launch_bounds__(kThreads) void bitlinear_gemv_kernel(
     float w_scale, int K, int KB, int N, int nquads, const float *residual, float *out) {
     constexpr int QPB = kWaves / KS;
     extern __shared__ uint4 s_a[];  // KB staged activation blocks (4-bit planes)
-    __shared__ float s_red[kWaves];
+    __shared__ float s_ss[kWaves], s_mx[kWaves];
     __shared__ int s_redi[kWaves];
     __shared__ int s_part[KS > 1 ? kWaves * 4 : 1];
 
@@ -91,9 +104,9 @@ __global__ __launch_bounds__(kThreads) void bitlinear_gemv_kernel(
 
     // (1) the row and the gains, (2) the first round of weights: all loads unconditional
     // (indices clamped), back to back
-    float v[kMaxBlocksPerThread][16], gm[kMaxBlocksPerThread][16];
+    float v[NB][16], gm[NB][16];
 #pragma unroll
-    for (int b = 0; b < kMaxBlocksPerThread; ++b) {
+    for (int b = 0; b < NB; ++b) {
         const int kb = min(tid + b * kThreads, kreal - 1);
         const float4 *xr = reinterpret_cast<const float4 *>(x) + kb * 4;
         const float4 *gr = reinterpret_cast<const float4 *>(gamma) + kb * 4;
@@ -126,40 +139,37 @@ __global__ __launch_bounds__(kThreads) void bitlinear_gemv_kernel(
     }
     __builtin_amdgcn_sched_barrier(0);
 
-    // normalise and quantise (every workgroup computes the same values in the same order)
-    float ss = 0.0f;
+    // One pass gives both statistics: sum v^2, and max |v * gamma| - rounding is monotone, so
+    // max_k |fl(t_k * r)| = fl(max_k |t_k| * r) for the positive factor r = inv_rms.  Every
+    // workgroup computes the same values in the same order.
+    float ss = 0.0f, mx = 0.0f;
 #pragma unroll
-    for (int b = 0; b < kMaxBlocksPerThread; ++b) {
+    for (int b = 0; b < NB; ++b) {
         const bool mine = tid + b * kThreads < kreal;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            v[b][e] = mine ? v[b][e] : 0.0f;
-            ss += v[b][e] * v[b][e];
+            const float a = mine ? v[b][e] : 0.0f;
+            ss += a * a;
+            v[b][e] = a * gm[b][e];
+            mx = fmaxf(mx, fabsf(v[b][e]));
         }
     }
-    ss = wave_sum_f(ss);
-    if (lane == 0) s_red[wave] = ss;
+    ss = wave_sum_lane63(ss);
+    mx = wave_max_lane63(mx);
+    if (lane == 63) {
+        s_ss[wave] = ss;
+        s_mx[wave] = mx;
+    }
     __syncthreads();
-    ss = (s_red[0] + s_red[1]) + (s_red[2] + s_red[3]);
+    ss = (s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3]);
+    mx = fmaxf(fmaxf(s_mx[0], s_mx[1]), fmaxf(s_mx[2], s_mx[3]));
     const float inv_rms = 1.0f / sqrtf(ss / (float)K + eps);
-    float amax = 0.0f;
-#pragma unroll
-    for (int b = 0; b < kMaxBlocksPerThread; ++b)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            v[b][e] = (v[b][e] * inv_rms) * gm[b][e];
-            amax = fmaxf(amax, fabsf(v[b][e]));
-        }
-    amax = wave_max_f(amax);
-    __syncthreads();
-    if (lane == 0) s_red[wave] = amax;
-    __syncthreads();
-    const float gmax = fmaxf(fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3])), 1e-5f);
+    const float gmax = fmaxf(mx * inv_rms, 1e-5f);
     const float inv = 127.0f / gmax;
     const float act_scale = gmax / 127.0f;
     int qsum = 0;
 #pragma unroll
-    for (int b = 0; b < kMaxBlocksPerThread; ++b) {
+    for (int b = 0; b < NB; ++b) {
         const int kb = tid + b * kThreads;
         uint32_t pk[4];
 #pragma unroll
@@ -167,7 +177,8 @@ __global__ __launch_bounds__(kThreads) void bitlinear_gemv_kernel(
             uint32_t word = 0;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                float r = rintf(v[b][4 * c + e] * inv);  // round half to even
+                const float y = v[b][4 * c + e] * inv_rms;
+                float r = rintf(y * inv);  // round half to even
                 r = fminf(fmaxf(r, -128.0f), 127.0f);
                 const int qi = (int)r;
                 qsum += qi;
@@ -177,8 +188,8 @@ __global__ __launch_bounds__(kThreads) void bitlinear_gemv_kernel(
         }
         if (kb < KB) s_a[kb] = to_nibble_planes(make_uint4(pk[0], pk[1], pk[2], pk[3]));  // zeros in the padding
     }
-    qsum = wave_sum_i(qsum);
-    if (lane == 0) s_redi[wave] = qsum;
+    qsum = wave_total_lane63(qsum);
+    if (lane == 63) s_redi[wave] = qsum;
     __syncthreads();
     const int rowsum = (s_redi[0] + s_redi[1]) + (s_redi[2] + s_redi[3]);
 
@@ -267,8 +278,12 @@ template <int KS, int L, bool SWIGLU>
 void launch(hipStream_t stream, const Args &a) {
     constexpr int QPB = kWaves / KS;
     dim3 grid((unsigned)((a.nquads + QPB - 1) / QPB));
-    bitlinear_gemv_kernel<KS, L, SWIGLU><<<grid, dim3(kThreads), (size_t)a.KB * 16, stream>>>(
-        a.x, a.gamma, a.eps, a.w4, a.w_scale, a.K, a.KB, a.N, a.nquads, a.residual, a.out);
+    if (a.K <= 16 * kThreads)
+        bitlinear_gemv_kernel<KS, L, SWIGLU, 1><<<grid, dim3(kThreads), (size_t)a.KB * 16, stream>>>(
+            a.x, a.gamma, a.eps, a.w4, a.w_scale, a.K, a.KB, a.N, a.nquads, a.residual, a.out);
+    else
+        bitlinear_gemv_kernel<KS, L, SWIGLU, 2><<<grid, dim3(kThreads), (size_t)a.KB * 16, stream>>>(
+            a.x, a.gamma, a.eps, a.w4, a.w_scale, a.K, a.KB, a.N, a.nquads, a.residual, a.out);
 }
 
 template <int KS, bool SWIGLU>

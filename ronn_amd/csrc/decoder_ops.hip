@@ -42,7 +42,7 @@ __global__ __launch_bounds__(kBlock) void embed_kernel(const float *__restrict__
 // One workgroup of 1024 threads per token:
 //   x = silu(gate) * up   when gate_up is given (SwiGLU computed on the way in), else
 //   x += delta            when delta is given (written back: the residual stream)
-//   y = (x * rsqrt(mean(x^2) + eps)) * gamma
+//   y = (x * gamma) * rsqrt(mean(x^2) + eps)
 //   g = max(max|y|, 1e-5); q = clamp(rne(y * (127/g)), -128, 127); scale = g/127; rowsum = sum q
 // With one token the kernel is a chain of memory round trips, so every load (row, delta,
 // gains) is issued before the first reduction and the row stays in registers.
@@ -52,7 +52,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_quant_kernel(
     float *__restrict__ x, const float *__restrict__ delta, const float *__restrict__ gate_up,
     const float *__restrict__ gamma, float eps, int H, int pitch, int8_t *__restrict__ q,
     float *__restrict__ act_scale, int32_t *__restrict__ rowsum) {
-    __shared__ float s_red[kNormThreads / 64];
+    __shared__ float s_red[kNormThreads / 64], s_redm[kNormThreads / 64];
     __shared__ int s_redi[kNormThreads / 64];
     const int m = blockIdx.x, tid = threadIdx.x;
     float v[kPer], gm[kPer];
@@ -85,30 +85,32 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_quant_kernel(
             }
         }
     }
-    float ss = 0.0f;
-#pragma unroll
-    for (int j = 0; j < kPer; ++j) ss += v[j] * v[j];
-    ss = wave_sum_f(ss);
-    if ((tid & 63) == 0) s_red[tid >> 6] = ss;
-    __syncthreads();
-    ss = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kNormThreads / 64; ++w) ss += s_red[w];
-    const float inv_rms = 1.0f / sqrtf(ss / (float)H + eps);
-    float amax = 0.0f;
+    // one pass for both statistics: sum x^2 and max |x * gamma| (rounding is monotone, so
+    // max_k |fl(t_k * r)| = fl(max_k |t_k| * r) for r = inv_rms > 0)
+    float ss = 0.0f, mx = 0.0f;
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
-        v[j] = (v[j] * inv_rms) * gm[j];
-        amax = fmaxf(amax, fabsf(v[j]));
+        ss += v[j] * v[j];
+        v[j] *= gm[j];
+        mx = fmaxf(mx, fabsf(v[j]));
     }
-    amax = wave_max_f(amax);
+    ss = wave_sum_f(ss);
+    mx = wave_max_f(mx);
+    if ((tid & 63) == 0) {
+        s_red[tid >> 6] = ss;
+        s_redm[tid >> 6] = mx;
+    }
     __syncthreads();
-    if ((tid & 63) == 0) s_red[tid >> 6] = amax;
-    __syncthreads();
-    amax = 0.0f;
+    ss = 0.0f, mx = 0.0f;
 #pragma unroll
-    for (int w = 0; w < kNormThreads / 64; ++w) amax = fmaxf(amax, s_red[w]);
-    const float gmax = fmaxf(amax, 1e-5f);
+    for (int w = 0; w < kNormThreads / 64; ++w) {
+        ss += s_red[w];
+        mx = fmaxf(mx, s_redm[w]);
+    }
+    const float inv_rms = 1.0f / sqrtf(ss / (float)H + eps);
+    const float gmax = fmaxf(mx * inv_rms, 1e-5f);
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) v[j] *= inv_rms;
     const float inv = 127.0f / gmax;
     int sum = 0;
     int8_t *qrow = q + (size_t)m * pitch;

@@ -11,11 +11,11 @@ from util import epilogue, exact_int_matmul, oracle_weights
 
 
 def rmsnorm_quant(x, gamma, eps):
-    """y = (x * rsqrt(mean(x^2) + eps)) * gamma, then per-token int8 quantisation."""
+    """y = (x * gamma) * rsqrt(mean(x^2) + eps), then per-token int8 quantisation."""
     x = x.astype(np.float32)
     ss = (x.astype(np.float64) ** 2).sum(axis=1) / x.shape[1]
     inv = (1.0 / np.sqrt(ss.astype(np.float32) + np.float32(eps))).astype(np.float32)
-    y = (x * inv[:, None]).astype(np.float32) * gamma.astype(np.float32)[None, :]
+    y = (x * gamma.astype(np.float32)[None, :]).astype(np.float32) * inv[:, None]
     q, s, rs = O.act_quant_i8(y.astype(np.float32))
     return y.astype(np.float32), q, s, rs
 

@@ -102,7 +102,10 @@ def test_bitlinear_gemv_single_launch(ctx, K, N, mode):
     # a code that flips by one step moves an output by one quantisation step of the product
     step = float(s[0]) * float(t.scale)
     assert np.abs(got - want).max() <= 4 * step + 1e-6 * np.abs(want).max()
-    assert (got == want).mean() > 0.5 or K <= 16 or mode == "swiglu"
+    # most outputs agree to the last bits: the device sums v^2 in f32 in its own order, so the
+    # activation scale may differ by an ulp (and with it every product), no more
+    ulps = np.abs(got - want) / np.maximum(np.abs(want), 1e-30)
+    assert np.median(ulps) <= 2.4e-7 or K <= 16 or mode == "swiglu"
 
 
 def test_embed_swiglu_argmax(ctx):

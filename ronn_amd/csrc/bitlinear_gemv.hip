@@ -20,9 +20,7 @@
 
 namespace {
 
-constexpr int kWaves = 4;
-constexpr int kThreads = kWaves * 64;
-constexpr int kMaxBlocksPerThread = 2;  // K <= 16 * 256 * 2 = 8192 (template NB: 1 up to 4096)
+constexpr int kMaxK = 8192;  // activations staged in LDS: 16 bytes per 16 k
 
 template <int CTRL, int ROWMASK>
 __device__ __forceinline__ int dpp_add(int v) {
@@ -75,13 +73,14 @@ __device__ __forceinline__ uint4 to_nibble_planes(uint4 a) {
 }
 
 // KS waves per column quad, L weight loads in flight per lane and round, SWIGLU input,
-// NB blocks of 16 activations per thread (K <= 4096 * NB).
-template <int KS, int L, bool SWIGLU, int NB>
-__global__ __launch_bounds__(kThreads) void bitlinear_gemv_kernel(
+// W waves per workgroup, NB blocks of 16 activations per thread (K <= 1024 * W * NB).
+template <int KS, int L, bool SWIGLU, int W, int NB>
+__global__ __launch_bounds__(W * 64) void bitlinear_gemv_kernel(
     const float *__restrict__ x,        // [K], or gate|up [2K] with SWIGLU
     const float *__restrict__ gamma,    // [K]
     float eps, const uint4 *__restrict__ w4,  // [nquads][KB]
     float w_scale, int K, int KB, int N, int nquads, const float *residual, float *out) {
+    constexpr int kWaves = W, kThreads = W * 64;
     constexpr int QPB = kWaves / KS;
     extern __shared__ uint4 s_a[];  // KB staged activation blocks (4-bit planes)
     __shared__ float s_ss[kWaves], s_mx[kWaves];
@@ -161,8 +160,12 @@ __global__ __launch_bounds__(kThreads) void bitlinear_gemv_kernel(
         s_mx[wave] = mx;
     }
     __syncthreads();
-    ss = (s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3]);
-    mx = fmaxf(fmaxf(s_mx[0], s_mx[1]), fmaxf(s_mx[2], s_mx[3]));
+    ss = 0.0f, mx = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kWaves; i += 4) {
+        ss += (s_ss[i] + s_ss[i + 1]) + (s_ss[i + 2] + s_ss[i + 3]);
+        mx = fmaxf(mx, fmaxf(fmaxf(s_mx[i], s_mx[i + 1]), fmaxf(s_mx[i + 2], s_mx[i + 3])));
+    }
     const float inv_rms = 1.0f / sqrtf(ss / (float)K + eps);
     const float gmax = fmaxf(mx * inv_rms, 1e-5f);
     const float inv = 127.0f / gmax;
@@ -191,7 +194,9 @@ __global__ __launch_bounds__(kThreads) void bitlinear_gemv_kernel(
     qsum = wave_total_lane63(qsum);
     if (lane == 63) s_redi[wave] = qsum;
     __syncthreads();
-    const int rowsum = (s_redi[0] + s_redi[1]) + (s_redi[2] + s_redi[3]);
+    int rowsum = 0;
+#pragma unroll
+    for (int i = 0; i < kWaves; ++i) rowsum += s_redi[i];
 
     int hi[4] = {0, 0, 0, 0}, lo[4] = {0, 0, 0, 0};
     auto consume = [&](const uint4(&wr)[L], int r0) {
@@ -274,16 +279,28 @@ struct Args {
     float *out;
 };
 
-template <int KS, int L, bool SWIGLU>
-void launch(hipStream_t stream, const Args &a) {
-    constexpr int QPB = kWaves / KS;
+template <int KS, int L, bool SWIGLU, int W>
+void launch_w(hipStream_t stream, const Args &a) {
+    constexpr int QPB = W / KS;
     dim3 grid((unsigned)((a.nquads + QPB - 1) / QPB));
-    if (a.K <= 16 * kThreads)
-        bitlinear_gemv_kernel<KS, L, SWIGLU, 1><<<grid, dim3(kThreads), (size_t)a.KB * 16, stream>>>(
+    if (a.K <= 1024 * W)
+        bitlinear_gemv_kernel<KS, L, SWIGLU, W, 1><<<grid, dim3(W * 64), (size_t)a.KB * 16, stream>>>(
             a.x, a.gamma, a.eps, a.w4, a.w_scale, a.K, a.KB, a.N, a.nquads, a.residual, a.out);
     else
-        bitlinear_gemv_kernel<KS, L, SWIGLU, 2><<<grid, dim3(kThreads), (size_t)a.KB * 16, stream>>>(
+        bitlinear_gemv_kernel<KS, L, SWIGLU, W, 2><<<grid, dim3(W * 64), (size_t)a.KB * 16, stream>>>(
             a.x, a.gamma, a.eps, a.w4, a.w_scale, a.K, a.KB, a.N, a.nquads, a.residual, a.out);
+}
+
+template <int KS, int L, bool SWIGLU>
+void launch(hipStream_t stream, const Args &a) {
+    // Every workgroup repeats the normalisation of the whole row: eight waves halve that
+    // work per thread and the number of workgroups re-reading the row.  It pays for long
+    // rows (K > 4096: one block per thread again) and for wide matrices (measured: 6912 x
+    // 2560 8.3 -> 5.6 us, 2560 x 13824 6.4 -> 6.1 us; 2560 x 2560 is faster with four).
+    if (a.K > 4096 || a.nquads >= 3072)
+        launch_w<KS, L, SWIGLU, 8>(stream, a);
+    else
+        launch_w<KS, L, SWIGLU, 4>(stream, a);
 }
 
 template <int KS, bool SWIGLU>
@@ -321,9 +338,9 @@ extern "C" int rbn_bitlinear_gemv_f32(rbn_ctx *ctx, const float *d_x, const floa
     RBN_REQUIRE((d_x != nullptr) != (d_gate_up != nullptr),
                 "rbn_bitlinear_gemv_f32 takes either d_x or d_gate_up");
     RBN_REQUIRE(d_gamma && d_tiled && d_out, "null pointer in rbn_bitlinear_gemv_f32");
-    RBN_REQUIRE(K >= 16 && K % 16 == 0 && K <= 16ull * kThreads * kMaxBlocksPerThread,
-                "rbn_bitlinear_gemv_f32 takes K %% 16 == 0, 16 <= K <= %d (got %llu)",
-                16 * kThreads * kMaxBlocksPerThread, (unsigned long long)K);
+    RBN_REQUIRE(K >= 16 && K % 16 == 0 && K <= (uint64_t)kMaxK,
+                "rbn_bitlinear_gemv_f32 takes K %% 16 == 0, 16 <= K <= %d (got %llu)", kMaxK,
+                (unsigned long long)K);
     RBN_REQUIRE(N > 0 && N <= (1ull << 30), "bad N in rbn_bitlinear_gemv_f32");
     const float *src = d_x ? d_x : d_gate_up;
     RBN_REQUIRE((((uintptr_t)src | (uintptr_t)d_gamma | (uintptr_t)d_tiled) & 15u) == 0,

@@ -15,17 +15,44 @@ namespace {
 
 constexpr int kBlock = 256;
 
+// Wave-wide reductions on the DPP cross-lane path (a few cycles per step, against a trip
+// through the LDS crossbar for a shuffle): quad_perm, row_ror within rows of 16 lanes,
+// row_bcast across rows; the total arrives in lane 63 and is read back as a wave-uniform
+// value.  Lanes outside a step's row mask see `old`.  All 64 lanes must be active.
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ int dpp_i(int old, int v) {
+    return __builtin_amdgcn_update_dpp(old, v, CTRL, ROWMASK, 0xf, false);
+}
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ float dpp_f(float old, float v) {
+    return __int_as_float(dpp_i<CTRL, ROWMASK>(__float_as_int(old), __float_as_int(v)));
+}
 __device__ __forceinline__ float wave_sum_f(float v) {
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    return v;
+    v += dpp_f<0xB1, 0xf>(0.0f, v);   // quad_perm [1,0,3,2]
+    v += dpp_f<0x4E, 0xf>(0.0f, v);   // quad_perm [2,3,0,1]
+    v += dpp_f<0x124, 0xf>(0.0f, v);  // row_ror:4
+    v += dpp_f<0x128, 0xf>(0.0f, v);  // row_ror:8
+    v += dpp_f<0x142, 0xA>(0.0f, v);  // row_bcast15
+    v += dpp_f<0x143, 0xC>(0.0f, v);  // row_bcast31
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 __device__ __forceinline__ float wave_max_f(float v) {
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    return v;
+    v = fmaxf(v, dpp_f<0xB1, 0xf>(v, v));
+    v = fmaxf(v, dpp_f<0x4E, 0xf>(v, v));
+    v = fmaxf(v, dpp_f<0x124, 0xf>(v, v));
+    v = fmaxf(v, dpp_f<0x128, 0xf>(v, v));
+    v = fmaxf(v, dpp_f<0x142, 0xA>(v, v));
+    v = fmaxf(v, dpp_f<0x143, 0xC>(v, v));
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 __device__ __forceinline__ int wave_sum_i(int v) {
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-    return v;
+    v += dpp_i<0xB1, 0xf>(0, v);
+    v += dpp_i<0x4E, 0xf>(0, v);
+    v += dpp_i<0x124, 0xf>(0, v);
+    v += dpp_i<0x128, 0xf>(0, v);
+    v += dpp_i<0x142, 0xA>(0, v);
+    v += dpp_i<0x143, 0xC>(0, v);
+    return __builtin_amdgcn_readlane(v, 63);
 }
 
 // x[m, :] = table[tokens[m], :]
@@ -292,6 +319,28 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
     if (p >= max_seq) p = max_seq - 1;
     const int nkeys = p + 1;
     const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
+    // The first block's keys and values do not depend on q: their loads go out before the
+    // rotary prologue and the barrier, whose latency they then cover.
+    const __half *kh = kcache + (size_t)h * max_seq * hd;
+    const __half *vh = vcache + (size_t)h * max_seq * hd;
+    const int kidx = lane >> 2, sub = lane & 3;
+    uint4 kr[4];
+    __half2 vr[16];
+    auto load_block = [&](int b) {
+        const int t0 = b * 16, last = max(nkeys - 1 - t0, 0);
+        const int t = t0 + min(kidx, last);
+        const uint4 *krow = reinterpret_cast<const uint4 *>(kh + (size_t)t * hd + sub * 32);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) kr[c] = krow[c];
+#pragma unroll
+        for (int j = 0; j < 16; ++j)
+            vr[j] = *reinterpret_cast<const __half2 *>(vh + (size_t)(t0 + min(j, last)) * hd + 2 * lane);
+    };
+    int b = sp * 4 + wave;
+    bool have = b * 16 < nkeys;
+    load_block(have ? b : 0);
+    __builtin_amdgcn_sched_barrier(0);
+
     if (tid < half) {
         const int i = tid;
         const float freq = powf(theta, -2.0f * (float)i / (float)hd);
@@ -317,21 +366,10 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
     }
     __syncthreads();
 
-    const __half *kh = kcache + (size_t)h * max_seq * hd;
-    const __half *vh = vcache + (size_t)h * max_seq * hd;
-    const int kidx = lane >> 2, sub = lane & 3;
     float run_max = -INFINITY, run_sum = 0.0f, o0 = 0.0f, o1 = 0.0f;
-    for (int b = sp * 4 + wave; b * 16 < nkeys; b += 4 * kSplits) {
+    while (have) {
         const int t0 = b * 16, last = nkeys - 1 - t0;  // last >= 0
         const int t = t0 + min(kidx, last);
-        const uint4 *krow = reinterpret_cast<const uint4 *>(kh + (size_t)t * hd + sub * 32);
-        uint4 kr[4];
-#pragma unroll
-        for (int c = 0; c < 4; ++c) kr[c] = krow[c];
-        __half2 vr[16];
-#pragma unroll
-        for (int j = 0; j < 16; ++j)
-            vr[j] = *reinterpret_cast<const __half2 *>(vh + (size_t)(t0 + min(j, last)) * hd + 2 * lane);
         float acc = 0.0f;
         const bool fresh = t == p;  // the row this launch adds: take it from LDS
 #pragma unroll
@@ -346,8 +384,8 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
                 acc = fmaf(f.y, s_q[d + 1], acc);
             }
         }
-        acc += __shfl_xor(acc, 1);
-        acc += __shfl_xor(acc, 2);
+        acc += dpp_f<0xB1, 0xf>(0.0f, acc);  // the four lanes of a key
+        acc += dpp_f<0x4E, 0xf>(0.0f, acc);
         const float s = kidx <= last ? acc : -INFINITY;
         const float new_max = fmaxf(run_max, wave_max_f(s));
         const float corr = __expf(run_max - new_max);  // 0 on the first block
@@ -365,6 +403,9 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
             o0 = fmaf(pj, v.x, o0);
             o1 = fmaf(pj, v.y, o1);
         }
+        b += 4 * kSplits;
+        have = b * 16 < nkeys;
+        if (have) load_block(b);
     }
     if (lane == 0) {
         s_m[wave] = run_max;

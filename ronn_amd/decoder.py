@@ -6,7 +6,7 @@ reference has no decoder (its BitNet provider stops at the matmul,
 crates/ronn-providers/src/bitnet/kernels.rs:134-178), so the layer formulas are the usual
 LLaMA / BitNet-b1.58 ones; tests/decoder_model.py restates them in numpy.
 
-A decode step is ~270 kernel launches; it reads the position and the previous token from
+A decode step is 124 kernel launches; it reads the position and the previous token from
 device memory, so it is captured once in a HIP graph and replayed per token.
 """
 from __future__ import annotations

@@ -342,8 +342,14 @@ def main():
                                     "GBps": bytes_per_launch / (ev1 * 1e-3) / 1e9,
                                     "note": "single 11 MiB weight buffer re-read from cache, not HBM"}
         del one
-        def kernel_for(m):
-            return "gemv" if m <= 3 else ("skinny_mfma" if m <= 64 else "gemm_mfma")
+        def kernel_for(m, k, n):
+            # the choice rbn_matmul_t2_i8 makes (csrc/gemm_mfma.hip)
+            if m <= 3:
+                return "gemv"
+            kn = k * n
+            if m <= 16 or (m <= 32 and kn < (1 << 27)) or (m <= 64 and kn < (1 << 25)):
+                return "skinny_mfma"
+            return "gemm_mfma"
 
         def sweep_over(shapes, ms, sigma):
             rows = []
@@ -352,7 +358,7 @@ def main():
                     w2 = wl if (m, k, n) == (M, K, N) else Workload(ctx, m, k, n, sigma, seed=3, mode=1)
                     ev, _, _ = time_graph(ctx, w2, ctx.matmul, 1500, 150)
                     b = gemv_bytes(m, k, n)
-                    rows.append({"M": m, "K": k, "N": n, "kernel": kernel_for(m), "us": ev * 1e3,
+                    rows.append({"M": m, "K": k, "N": n, "kernel": kernel_for(m, k, n), "us": ev * 1e3,
                                  "GBps": b / (ev * 1e-3) / 1e9,
                                  "frac_hbm_peak": b / (ev * 1e-3) / 1e9 / HBM_PEAK_GBS})
                     if w2 is not wl:

@@ -25,14 +25,15 @@ struct rbn_ctx {
     size_t ws_bytes = 0;
     // Pinned host mailbox for the few scalars that come back from the device.
     void *mailbox = nullptr;
-    // Split-k workspace of the small-batch matmul: RBN_SPLITK_TILES partial tiles of
-    // 16 x 64 int32 and one ticket counter per column group.  Allocated once with the
+    // Split-k workspace of the matmuls: RBN_SPLITK_TILES partial tiles of 16 x 64 int32
+    // (the prefill kernel takes sixteen of them per 64 x 256 partial) and one ticket counter
+    // per output tile.  Allocated once with the
     // context and never moved, so launches captured in a HIP graph stay valid.
     void *splitk_partials = nullptr;
     unsigned *splitk_tickets = nullptr;
 };
 
-constexpr int RBN_SPLITK_TILES = 4096;   // 16 MiB
+constexpr int RBN_SPLITK_TILES = 16384;  // 64 MiB
 constexpr int RBN_SPLITK_GROUPS = 1024;
 
 // Records `fmt...` as the calling thread's last error and returns `code`.

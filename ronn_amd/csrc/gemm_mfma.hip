@@ -81,8 +81,8 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
     const float *__restrict__ act_scale,  // [M]
     const int32_t *__restrict__ rowsum,   // [M]
     const uint4 *__restrict__ wt,         // tiled: uint4 index quad * KB + kb
-    float w_scale, int M, int Kpad, int N, int nquads, int m_tiles, int n_tiles,
-    int32_t *__restrict__ acc_out, float *__restrict__ out) {
+    float w_scale, int M, int Kpad, int N, int nquads, int m_tiles, int n_tiles, int splits,
+    int32_t *partials, unsigned *tickets, int32_t *__restrict__ acc_out, float *__restrict__ out) {
     // Ring of three stages in one array (units of 16 bytes): weights of stage s at
     // s * kBUnits, activations at 3 * kBUnits + s * kAUnits.
     constexpr int TM = 64 * MT;                  // rows of the tile
@@ -92,6 +92,7 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
     __shared__ __attribute__((aligned(16))) uint4 smem[3 * (kAUnits + kBUnits)];
     __shared__ float s_scale[TM];
     __shared__ int s_rowsum[TM];
+    __shared__ int s_last;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -101,15 +102,22 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
 
     // XCD-aware numbering: consecutive workgroups land on consecutive XCDs; give each XCD
     // a band of m tiles and let it walk the n tiles.
+    // With splits > 1 (few tiles, see the launch) `splits` consecutive workgroups share a
+    // tile and take consecutive ranges of K steps.
+    int tile = blockIdx.x, split = 0;
+    if (splits > 1) {
+        tile = blockIdx.x / splits;
+        split = blockIdx.x - tile * splits;
+    }
     int bm, bn;
-    if ((m_tiles & 7) == 0) {
+    if ((m_tiles & 7) == 0 && splits == 1) {
         const int per = m_tiles >> 3;
-        const int xcd = blockIdx.x & 7, i = blockIdx.x >> 3;
+        const int xcd = tile & 7, i = tile >> 3;
         bm = xcd * per + i % per;
         bn = i / per;
     } else {
-        bm = blockIdx.x % m_tiles;
-        bn = blockIdx.x / m_tiles;
+        bm = tile % m_tiles;
+        bn = tile / m_tiles;
     }
     const int m0 = bm * TM, n0 = bn * BN;
     const int q0 = n0 >> 2;
@@ -133,7 +141,7 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
     // slot holds segment (or k-block) slot ^ ((row >> 1) & 7) of that row.
     const int sub = lane >> 3;
     // a workgroup-uniform base (scalar registers) plus a 32-bit byte offset per lane
-    const int8_t *a_base = q + (size_t)m0 * Kpad;
+    const int8_t *a_base = q + (size_t)m0 * Kpad;  // advanced to this workgroup's first K step below
     uint32_t a_lane[2 * MT];
 #pragma unroll
     for (int j = 0; j < 2 * MT; ++j) {
@@ -149,7 +157,13 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
         const int kb = (lane & 7) ^ ((lquad >> 1) & 7);
         b_lane[j] = ((uint32_t)(min(q0 + lquad, nquads - 1) - q0) * (uint32_t)KB + kb) * 16;
     }
-    const int iters = Kpad / BK;
+    // this workgroup's K steps: [it_lo, it_lo + iters)
+    const int iters_all = Kpad / BK;
+    const int per_split = (iters_all + splits - 1) / splits;
+    const int it_lo = split * per_split;
+    const int iters = min(per_split, iters_all - it_lo);  // >= 1 (the launch sees to it)
+    a_base += (size_t)it_lo * BK;
+    b_base += (size_t)it_lo * (BK / 16);
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr)smem;
     auto issue = [&](int it, int stage) {
         const int kk = min(it, iters - 1);  // past the end: reload the last step, never read
@@ -275,6 +289,62 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
     if (it + 1 < iters) kstep(std::integral_constant<int, 1>{}, it + 1);
     __builtin_amdgcn_s_waitcnt(kWaitVm0);  // no load may still be writing LDS at exit
 
+    if constexpr (MT == 1) {
+        if (splits > 1) {
+            // Partial tiles meet in the workspace: every workgroup publishes its accumulators
+            // (register r of lane l of wave w at [(r * 4 + w) * 64 + l]) with device-scope
+            // stores, waits for them, and draws a ticket; the last of a tile adds the others'
+            // (integer sums: any order, same bits) and goes on to the epilogue.  Nobody waits
+            // for anybody.  The pointer is walked in a register the compiler cannot see
+            // through: folded into 64 constant offsets it costs 64 scalar register pairs.
+            // Register pair i of lane l of wave w sits at 64-bit index (i * 4 + w) * 64 + l.
+            // The lane offset is kept opaque to the compiler, which otherwise folds the 32
+            // positions into as many scalar register pairs.
+            constexpr size_t kPartialBytes = (size_t)64 * kThreads * 4;
+            char *mine = reinterpret_cast<char *>(partials) + ((size_t)tile * splits + split) * kPartialBytes;
+            uint32_t off = (uint32_t)(wave * 64 + lane) * 8;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) {
+                    const unsigned long long pair = (unsigned)acc[0][j][r] |
+                                                    ((unsigned long long)(unsigned)acc[0][j][r + 1] << 32);
+                    __hip_atomic_store(reinterpret_cast<unsigned long long *>(mine + off), pair,
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    off += kThreads * 8;
+                    asm volatile("" : "+v"(off));
+                }
+            __builtin_amdgcn_s_waitcnt(kWaitVm0);
+            __syncthreads();
+            if (tid == 0) {
+                const unsigned ticket = atomicAdd(&tickets[tile], 1u);
+                const int is_last = ticket == (unsigned)splits - 1;
+                if (is_last) atomicExch(&tickets[tile], 0u);  // ready for the next launch
+                s_last = is_last;
+            }
+            __syncthreads();
+            if (!s_last) return;
+            for (int s2 = 0; s2 < splits; ++s2) {
+                if (s2 == split) continue;
+                const char *theirs =
+                    reinterpret_cast<const char *>(partials) + ((size_t)tile * splits + s2) * kPartialBytes;
+                off = (uint32_t)(wave * 64 + lane) * 8;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int r = 0; r < 16; r += 2) {
+                        const unsigned long long pair =
+                            __hip_atomic_load(reinterpret_cast<const unsigned long long *>(theirs + off),
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        acc[0][j][r] += (int)(unsigned)pair;
+                        acc[0][j][r + 1] += (int)(unsigned)(pair >> 32);
+                        off += kThreads * 8;
+                        asm volatile("" : "+v"(off));
+                    }
+            }
+        }
+    }
+
     // epilogue: lane owns columns 4*quad .. 4*quad+3 (tile j -> column 4*quad + j) and rows
     // 8*(r/4) + 4*(lane/32) + r%4 of each 32-row tile
     const int col0 = n0 + fquad * 4;
@@ -339,14 +409,30 @@ extern "C" int rbn_gemm_t2_i8_mfma(rbn_ctx *ctx, const int8_t *d_q, const float 
     const int m_tiles = (int)((M + (low ? 63 : 127)) / (low ? 64 : 128));
     const uint64_t tiles = (uint64_t)m_tiles * n_tiles;
     RBN_REQUIRE(tiles <= 0x7fffffffull, "too many tiles");
+    // Very few tiles and a long K: split K over up to four workgroups per tile.  The parts
+    // meet through memory (64 KiB per partial tile, device-scope accesses), which costs about
+    // as much as ten K steps: measured, it pays up to ~96 tiles with at least sixteen K steps
+    // per part (6912 x 2560, M = 512: 26 -> 20 us; 11008 x 4096, M = 64: 39 -> 20 us) and
+    // loses beyond (4096 x 11008, M = 256: 18 -> 23 us).
+    int splits = 1;
+    if (low && tiles <= 96) {
+        const int iters = Kpad / BK;
+        const uint64_t room = 3ull * (uint64_t)ctx->props.multiProcessorCount;
+        while (splits < 4 && tiles * (splits + 1) <= room && iters / (splits + 1) >= 16) ++splits;
+        while (splits > 1 && (splits - 1) * ((iters + splits - 1) / splits) >= iters) --splits;
+        if (tiles > (uint64_t)RBN_SPLITK_GROUPS || tiles * splits * 16 > (uint64_t)RBN_SPLITK_TILES)
+            splits = 1;
+    }
+    const unsigned grid = (unsigned)(tiles * splits);
     if (low)
-        gemm_t2_i8_mfma_kernel<1><<<dim3((unsigned)tiles), dim3(kThreads), 0, ctx->stream>>>(
+        gemm_t2_i8_mfma_kernel<1><<<dim3(grid), dim3(kThreads), 0, ctx->stream>>>(
             d_q, d_act_scale, d_rowsum, (const uint4 *)d_tiled, w_scale, (int)M, Kpad, (int)N,
-            nquads, m_tiles, n_tiles, d_acc, d_out);
+            nquads, m_tiles, n_tiles, splits, (int32_t *)ctx->splitk_partials, ctx->splitk_tickets,
+            d_acc, d_out);
     else
-        gemm_t2_i8_mfma_kernel<2><<<dim3((unsigned)tiles), dim3(kThreads), 0, ctx->stream>>>(
+        gemm_t2_i8_mfma_kernel<2><<<dim3(grid), dim3(kThreads), 0, ctx->stream>>>(
             d_q, d_act_scale, d_rowsum, (const uint4 *)d_tiled, w_scale, (int)M, Kpad, (int)N,
-            nquads, m_tiles, n_tiles, d_acc, d_out);
+            nquads, m_tiles, n_tiles, 1, nullptr, nullptr, d_acc, d_out);
     RBN_HIP(hipGetLastError());
     return RBN_OK;
 }
@@ -355,11 +441,16 @@ extern "C" int rbn_matmul_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_
                                 const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
                                 uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc,
                                 float *d_out) {
-    // measured crossover: the dot-instruction GEMV wins up to three tokens
+    // measured crossovers: the dot-instruction GEMV wins up to three tokens; the streaming
+    // small-batch kernel up to 32 tokens (16 on very large matrices) and, on small matrices,
+    // up to its limit of 64; the tiled kernel beyond
     if (M <= 3)
         return rbn_gemv_t2_i8(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N, d_acc,
                               d_out);
-    if (M <= RBN_SKINNY_MAX_M)
+    const uint64_t kn = K * N;
+    const bool skinny = M <= 16 || (M <= 32 && kn < (1ull << 27)) ||
+                        (M <= RBN_SKINNY_MAX_M && kn < (1ull << 25));
+    if (skinny)
         return rbn_gemm_t2_i8_skinny(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N,
                                      d_acc, d_out);
     return rbn_gemm_t2_i8_mfma(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N, d_acc,

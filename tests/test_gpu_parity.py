@@ -306,6 +306,20 @@ def test_gemm_mfma_small(ctx, M, K, N):
     check_against_oracle(x, w, *res, literal=(M * K * N <= 1 << 23))
 
 
+@pytest.mark.parametrize("M,K,N", [(100, 1664, 600), (64, 8192, 1024), (300, 2560, 2560), (129, 1100, 4000),
+                                   (65, 640, 300)])
+def test_gemm_mfma_split_k(ctx, M, K, N):
+    # few tiles: the 64-row kernel splits K over up to four workgroups per tile, which meet
+    # through the context's workspace (13 K steps -> parts of 5, 5 and 3); run twice, the
+    # second launch finds the tickets as the first one left them
+    say("gemm split k", M, K, N)
+    x = synth_normal(0x5EED000B + M, 1.0, (M, K))
+    w = synth_normal(0x5EED100B + N, 0.02, (K, N))
+    for _ in range(2):
+        res = run_matmul(ctx, ctx.gemm, x, w)
+        check_against_oracle(x, w, *res, literal=False)
+
+
 @pytest.mark.parametrize("M,K,N", [(2000, 128, 11016), (1030, 256, 15000), (1100, 384, 15000),
                                    (2048, 512, 11008)])
 def test_gemm_mfma_more_than_one_round(ctx, M, K, N):

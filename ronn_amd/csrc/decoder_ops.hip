@@ -292,6 +292,191 @@ __global__ __launch_bounds__(kWaves * 64) void attention_kernel(
     }
 }
 
+// Attention of a prompt on the f16 matrix cores: one workgroup per (block of 32 tokens, head),
+// its four waves take every fourth block of 32 keys, keep an online softmax each and meet
+// through LDS at the end.  hd == 128.
+//  * Scores transposed, S^T = K . Q^T (v_mfma_f32_32x32x16_f16, A = 32 keys x 16 dims read as
+//    one 16-byte piece of a key row per lane, B = Q^T): a lane then holds ONE token (column
+//    lane % 32) and 16 of the 32 keys, so the softmax is lane-local but for one exchange with
+//    lane ^ 32.  The same lane layout comes out of O^T = V^T . P^T, so the running rescale of
+//    O is lane-local too, and P^T is already in B-operand form: MFMA step s multiplies the
+//    lane's own probabilities 8s .. 8s+7, i.e. keys 8(2s + e/4) + 4(lane/32) + e%4.
+//  * V^T . P^T needs values with the key index contiguous per lane: the wave stages its 32
+//    value rows in LDS (row pitch 136 halves: the two lane halves read rows four apart, on
+//    disjoint banks) and gathers the eight keys of a slot set with 16-bit reads.
+//  * f32-grade accuracy from f16 matrix cores: K and V are f16 already; q (scaled) and the
+//    probabilities go in as hi + lo f16 pairs, two MFMAs each, accumulated in f32.
+//  * Rows past the last key of the prompt are never loaded (indices clamp to it: everything
+//    up to there has been written), so masked keys multiply finite values by zero.
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+constexpr int kVPitch = 136;  // halves per staged value row
+__global__ __launch_bounds__(256) void attention_mfma_kernel(
+    const float *__restrict__ qkv, const int32_t *__restrict__ pos0, int M, int heads,
+    const __half *__restrict__ kcache, const __half *__restrict__ vcache, int max_seq,
+    float *__restrict__ out) {
+    constexpr int hd = 128;
+    __shared__ __attribute__((aligned(16))) _Float16 s_v[4][32 * kVPitch];  // later: the exchange
+    __shared__ float s_ml[4][2][64];
+    const int nqb = (M + 31) >> 5;
+    const int qb = nqb - 1 - (int)(blockIdx.x / heads);  // the long blocks first
+    const int h = blockIdx.x % heads;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int j = lane & 31, g = lane >> 5;
+    const int HD = heads * hd;
+    const int p0 = pos0[0];
+    const int m = min(qb * 32 + j, M - 1);            // this lane's token (clamped: never stored twice)
+    const int pj = min(p0 + m, max_seq - 1);          // its position = its last key
+    const int last_key = min(p0 + M - 1, max_seq - 1);  // last row of the caches that is known to be written
+    const int blk_keys = min(p0 + qb * 32 + 31, last_key) + 1;
+    const int nkb = (blk_keys + 31) >> 5;
+
+    // Q^T operand: dims 16 kk + 8 g + e of token j, scaled, as f16 hi + lo
+    v8h qhi[8], qlo[8];
+    {
+        const float scale = 0.08838834764831845f;  // 1 / sqrt(128)
+        const float *qrow = qkv + (size_t)m * 3 * HD + h * hd + 8 * g;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+            const float4 a = *reinterpret_cast<const float4 *>(qrow + 16 * kk);
+            const float4 b = *reinterpret_cast<const float4 *>(qrow + 16 * kk + 4);
+            const float f[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float v = f[e] * scale;
+                const _Float16 hi = (_Float16)v;
+                qhi[kk][e] = hi;
+                qlo[kk][e] = (_Float16)(v - (float)hi);
+            }
+        }
+    }
+
+    const __half *kh = kcache + (size_t)h * max_seq * hd;
+    const __half *vh = vcache + (size_t)h * max_seq * hd;
+    _Float16 *sv = s_v[wave];
+    float run_max = -INFINITY, run_sum = 0.0f;
+    v16f ot[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ot[nt][r] = 0.0f;
+
+    for (int kb = wave; kb < nkb; kb += 4) {
+        const int t0 = kb * 32;
+        // key rows (A operand of the scores) and the staging of the value rows
+        const uint4 *krow = reinterpret_cast<const uint4 *>(kh + (size_t)min(t0 + j, last_key) * hd + 8 * g);
+        uint4 kr[8];
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) kr[kk] = krow[2 * kk];
+        uint4 vstage[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const int idx = c * 64 + lane, row = idx >> 4, col = idx & 15;
+            vstage[c] = *reinterpret_cast<const uint4 *>(vh + (size_t)min(t0 + row, last_key) * hd + 8 * col);
+        }
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            const int idx = c * 64 + lane, row = idx >> 4, col = idx & 15;
+            *reinterpret_cast<uint4 *>(sv + row * kVPitch + 8 * col) = vstage[c];
+        }
+        // S^T: keys 8b + 4g + r (register 4b + r) of token j
+        v16f st;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) st[r] = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < 8; ++kk) {
+            const v8h ka = __builtin_bit_cast(v8h, kr[kk]);
+            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qhi[kk], st, 0, 0, 0);
+            st = __builtin_amdgcn_mfma_f32_32x32x16_f16(ka, qlo[kk], st, 0, 0, 0);
+        }
+        float blk_max = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int t = t0 + 8 * (r >> 2) + 4 * g + (r & 3);
+            st[r] = t <= pj ? st[r] : -INFINITY;
+            blk_max = fmaxf(blk_max, st[r]);
+        }
+        blk_max = fmaxf(blk_max, __shfl_xor(blk_max, 32));
+        const float new_max = fmaxf(run_max, blk_max);
+        const float ref = new_max == -INFINITY ? 0.0f : new_max;  // nothing valid yet: all p = 0
+        const float corr = __expf(run_max - ref);
+        float psum = 0.0f;
+        v8h phi[2], plo[2];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float pr = __expf(st[r] - ref);
+            psum += pr;
+            const _Float16 hi = (_Float16)pr;
+            phi[r >> 3][r & 7] = hi;
+            plo[r >> 3][r & 7] = (_Float16)(pr - (float)hi);
+        }
+        psum += __shfl_xor(psum, 32);
+        run_sum = run_sum * corr + psum;
+        run_max = new_max;
+        // O^T: dims 32 nt + (8b + 4g + r) of token j
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ot[nt][r] *= corr;
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+                v8h vt;
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    vt[e] = sv[(8 * (2 * s2 + (e >> 2)) + 4 * g + (e & 3)) * kVPitch + 32 * nt + j];
+                ot[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vt, phi[s2], ot[nt], 0, 0, 0);
+                ot[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vt, plo[s2], ot[nt], 0, 0, 0);
+            }
+        }
+    }
+
+    // The four waves' states meet pairwise: 1 -> 0 and 3 -> 2, then 2 -> 0.  The exchange
+    // area reuses the value staging (everybody is past its loop after the first barrier).
+    float *xch = reinterpret_cast<float *>(&s_v[0][0]);  // 2 x 64 registers x 64 lanes
+    auto publish = [&](int slot) {
+        float *dst = xch + slot * (64 * 64);
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dst[(nt * 16 + r) * 64 + lane] = ot[nt][r];
+        s_ml[slot][0][lane] = run_max;
+        s_ml[slot][1][lane] = run_sum;
+    };
+    auto merge = [&](int slot) {
+        const float *src = xch + slot * (64 * 64);
+        const float m2 = s_ml[slot][0][lane], l2 = s_ml[slot][1][lane];
+        const float mx = fmaxf(run_max, m2);
+        const float ref = mx == -INFINITY ? 0.0f : mx;
+        const float c1 = __expf(run_max - ref), c2 = __expf(m2 - ref);
+        run_sum = c1 * run_sum + c2 * l2;
+        run_max = mx;
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ot[nt][r] = c1 * ot[nt][r] + c2 * src[(nt * 16 + r) * 64 + lane];
+    };
+    static_assert(sizeof(s_v) >= 2 * 64 * 64 * sizeof(float), "the exchange area must fit the staging");
+    __syncthreads();
+    if (wave & 1) publish(wave >> 1);
+    __syncthreads();
+    if (!(wave & 1)) merge(wave >> 1);
+    __syncthreads();
+    if (wave == 2) publish(0);
+    __syncthreads();
+    if (wave != 0) return;
+    merge(0);
+    if (qb * 32 + j >= M) return;  // a clamped duplicate of the last token
+    const float inv = 1.0f / run_sum;
+    float *orow = out + (size_t)m * HD + h * hd + 4 * g;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+            *reinterpret_cast<float4 *>(orow + 32 * nt + 8 * b) =
+                make_float4(ot[nt][4 * b] * inv, ot[nt][4 * b + 1] * inv, ot[nt][4 * b + 2] * inv,
+                            ot[nt][4 * b + 3] * inv);
+}
+
 // Decoding one token: rotary embedding, cache store and attention in one launch, spread
 // over kSplits workgroups per head so that many CUs pull the cache at once.
 //  * Every workgroup rotates q (and the new k) itself; split 0 also writes the new k and v
@@ -592,8 +777,14 @@ int rbn_attention_f16kv(rbn_ctx *ctx, const float *d_qkv, const int32_t *d_pos0,
                 (unsigned long long)head_dim);
     RBN_REQUIRE(M > 0 && heads > 0 && M * heads < (1ull << 31) && max_seq > 0 && max_seq < (1u << 24),
                 "bad sizes in rbn_attention_f16kv");
-    // a single token (decode) gets more waves per head: only `heads` workgroups run
-    if (M == 1)
+    // a single token (decode) gets more waves per head: only `heads` workgroups run;
+    // prompts of at least 32 tokens go to the matrix cores
+    if (M >= 32) {
+        const uint64_t blocks = (M + 31) / 32 * heads;
+        attention_mfma_kernel<<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>(
+            d_qkv, d_pos0, (int)M, (int)heads, (const __half *)d_kcache, (const __half *)d_vcache,
+            (int)max_seq, d_out);
+    } else if (M == 1)
         attention_kernel<8><<<dim3((unsigned)(M * heads)), dim3(8 * 64), 0, ctx->stream>>>(
             d_qkv, d_pos0, (int)heads, (const __half *)d_kcache, (const __half *)d_vcache, (int)max_seq, d_out);
     else

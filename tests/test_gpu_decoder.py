@@ -129,8 +129,12 @@ def test_embed_swiglu_argmax(ctx):
     assert d_pos.download(np.int32, 1)[0] == 8
 
 
-@pytest.mark.parametrize("M,pos0,heads", [(1, 0, 2), (1, 130, 3), (6, 0, 2), (5, 250, 2), (1, 1023, 1)])
+@pytest.mark.parametrize("M,pos0,heads", [(1, 0, 2), (1, 130, 3), (6, 0, 2), (5, 250, 2), (1, 1023, 1),
+                                          (32, 0, 1), (64, 0, 2), (100, 37, 3), (33, 990, 1), (512, 0, 2),
+                                          (200, 300, 1)])
 def test_rope_store_and_attention(ctx, M, pos0, heads):
+    # from 32 tokens on the attention runs on the f16 matrix cores (same tolerance: q and
+    # the probabilities enter as hi + lo pairs)
     hd, max_seq, theta = 128, 1024, 10000.0
     A = heads * hd
     rng = np.random.default_rng(M * 1000 + pos0)

@@ -174,24 +174,30 @@ __global__ __launch_bounds__(kBlock) void rope_kv_store_kernel(
     const int pos = pos0[0] + m;
     const int HD = heads * hd, half = hd >> 1;
     float *qrow = qkv + (size_t)m * 3 * HD;
-    for (int idx = threadIdx.x; idx < heads * half; idx += kBlock) {
-        const int h = idx / half, i = idx - h * half;
+    // A thread keeps one pair index i (its angle is computed once) and walks the heads:
+    // `groups` threads share an i and take every groups-th head.
+    const int groups = kBlock >= half ? kBlock / half : 1;
+    const int group = kBlock >= half ? (int)threadIdx.x / half : 0;
+    if (group >= groups) return;  // left-over threads when half does not divide the block
+    for (int i = (int)threadIdx.x % half; i < half; i += kBlock) {  // one pass unless half > kBlock
         const float freq = powf(theta, -2.0f * (float)i / (float)hd);
         float sn, cs;
         sincosf((float)pos * freq, &sn, &cs);
-        float *qh = qrow + h * hd, *kh = qrow + HD + h * hd;
-        const float *vh = qrow + 2 * HD + h * hd;
-        const float q0 = qh[i], q1 = qh[i + half];
-        qh[i] = q0 * cs - q1 * sn;
-        qh[i + half] = q1 * cs + q0 * sn;
-        const float k0 = kh[i], k1 = kh[i + half];
-        const float r0 = k0 * cs - k1 * sn, r1 = k1 * cs + k0 * sn;
-        if (pos < max_seq) {
-            const size_t c = ((size_t)h * max_seq + pos) * hd;
-            kcache[c + i] = __float2half_rn(r0);
-            kcache[c + i + half] = __float2half_rn(r1);
-            vcache[c + i] = __float2half_rn(vh[i]);
-            vcache[c + i + half] = __float2half_rn(vh[i + half]);
+        for (int h = group; h < heads; h += groups) {
+            float *qh = qrow + h * hd, *kh = qrow + HD + h * hd;
+            const float *vh = qrow + 2 * HD + h * hd;
+            const float q0 = qh[i], q1 = qh[i + half];
+            qh[i] = q0 * cs - q1 * sn;
+            qh[i + half] = q1 * cs + q0 * sn;
+            const float k0 = kh[i], k1 = kh[i + half];
+            const float r0 = k0 * cs - k1 * sn, r1 = k1 * cs + k0 * sn;
+            if (pos < max_seq) {
+                const size_t c = ((size_t)h * max_seq + pos) * hd;
+                kcache[c + i] = __float2half_rn(r0);
+                kcache[c + i + half] = __float2half_rn(r1);
+                vcache[c + i] = __float2half_rn(vh[i]);
+                vcache[c + i + half] = __float2half_rn(vh[i + half]);
+            }
         }
     }
 }

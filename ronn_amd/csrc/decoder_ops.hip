@@ -670,13 +670,33 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
     __shared__ int s_i[16];
     float best = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < n; i += 1024) {
-        const float x = v[i];
+    auto take = [&](float x, int i) {
         if (x > best || (x == best && i < bi)) {
             best = x;
             bi = i;
         }
+    };
+    // batches of 32 values per thread (eight 16-byte loads, all issued before the first
+    // comparison: one memory round trip per batch instead of one per value)
+    int base = 0;
+    if ((reinterpret_cast<uintptr_t>(v) & 15u) == 0) {
+        const int n4 = n & ~3;
+        for (; base < n4; base += 32 * 1024) {
+            float4 x[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int i = base + 4 * ((int)threadIdx.x + 1024 * j);
+                x[j] = *reinterpret_cast<const float4 *>(v + min(i, n4 - 4));
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int i = base + 4 * ((int)threadIdx.x + 1024 * j);
+                if (i < n4) take(x[j].x, i), take(x[j].y, i + 1), take(x[j].z, i + 2), take(x[j].w, i + 3);
+            }
+        }
+        base = n4;
     }
+    for (int i = base + threadIdx.x; i < n; i += 1024) take(v[i], i);
     for (int off = 32; off > 0; off >>= 1) {
         const float ob = __shfl_xor(best, off);
         const int oi = __shfl_xor(bi, off);

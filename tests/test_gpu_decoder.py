@@ -127,6 +127,14 @@ def test_embed_swiglu_argmax(ctx):
     assert d_i.download(np.int32, 1)[0] == 77 and d_hist.download(np.int32, 16)[3] == 77
     check(ctx.lib.rbn_add_i32(ctx.handle, d_pos.ptr, 5))
     assert d_pos.download(np.int32, 1)[0] == 8
+    # sizes around the batches of 16-byte loads, the maximum in the scalar tail, unaligned input
+    for n, where, shift in ((1, 0, 0), (5, 4, 0), (1000, 999, 0), (4099, 4098, 0), (40001, 32769, 0),
+                            (70000, 69999, 0), (5000, 17, 1), (32768, 32767, 0)):
+        w = synth_normal(24 + n, 1.0, (n + shift,))
+        w[shift + where] = w.max() + 1
+        d_w = ctx.to_device(w)
+        check(ctx.lib.rbn_argmax_f32(ctx.handle, d_w.ptr + 4 * shift, n, d_i.ptr, None, None))
+        assert d_i.download(np.int32, 1)[0] == where, (n, where, shift)
 
 
 @pytest.mark.parametrize("M,pos0,heads", [(1, 0, 2), (1, 130, 3), (6, 0, 2), (5, 250, 2), (1, 1023, 1),

@@ -319,7 +319,7 @@ def main():
                    "compute_units": info["compute_units"], "clock_mhz": info["clock_khz"] / 1000.0},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": GEMV_HEADLINE_TRAFFIC_BYTES,
-                     "kernel": "gemv_t2_i8_kernel<1,8>", "bytes_per_launch": bytes_per_launch,
+                     "kernel": "gemv_t2_i8_kernel<1, 1, 4>", "bytes_per_launch": bytes_per_launch,
                      "us_per_launch": ev_ms * 1e3},
     }
 

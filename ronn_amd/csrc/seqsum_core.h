@@ -166,7 +166,7 @@ SEQ_HD uint32_t seq_apply(SeqMap m, uint32_t k) { return k + ((k & 1u) ? m.d1 : 
 // more of every term in a higher binade) the window just ends early and the next one
 // continues with a fresh rate; blocks past a crossing are the only wasted reads.
 #include <math.h>
-static inline uint64_t seq_next_window(uint64_t pos, uint64_t total_blocks, double s_now, double rate) {
+SEQ_HD uint64_t seq_next_window(uint64_t pos, uint64_t total_blocks, double s_now, double rate) {
     uint64_t win = pos + pos / 2;
     if (rate > 0.0 && s_now > 0.0 && isfinite(s_now)) {
         int e = 0;

@@ -151,23 +151,34 @@ __global__ __launch_bounds__(kBlock) void abs_sum_tree_final_kernel(
 // ---------------------------------------------------------------------------
 // Strict mode: the kernels of the exact sequential sum (see seqsum_core.h).
 // ---------------------------------------------------------------------------
+// The state of a sum lives in device memory and drives the kernels themselves, so that several
+// windows can be queued without the host in between; the kernel that ends a window mirrors it
+// into pinned host memory.
 struct SeqState {
-    uint32_t s_bits;       // current sum S as f32 bits (S >= 0)
-    uint32_t cross_block;  // window-relative block in which S leaves its binade, or ~0u
-    uint32_t k;            // integer state entering cross_block, or after the window
-    uint32_t next_rel;     // window-relative block at which the next window starts
-    uint32_t saw_nan;      // set by any_nan_kernel
-    uint32_t pad[3];
+    uint32_t s_bits;    // current sum S as f32 bits (S >= 0)
+    uint32_t win;       // blocks in the window that starts at `pos`
+    uint64_t pos;       // blocks already folded into S
+    uint32_t done;      // all blocks folded, or S no longer finite: queued kernels just return
+    uint32_t error;     // a window made no progress (internal error)
+    uint32_t saw_nan;   // set by any_nan_kernel
+    uint32_t pad;
 };
 
 // One SeqMap per block of 4096 elements, valid for a state of biased exponent `es`.
+// The window and the exponent come from the state; the grid strides over the window's blocks.
 __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
-    const float *__restrict__ x, uint64_t first, uint64_t n, uint32_t es, int use_mask,
-    float thr, SeqMap *__restrict__ maps) {
+    const float *__restrict__ x, uint64_t n, int use_mask, float thr,
+    const SeqState *__restrict__ state, SeqMap *__restrict__ maps) {
     __shared__ SeqMap s_wave[kBlock / 64];
-    uint64_t base = first + (uint64_t)blockIdx.x * kSeqTile + (uint64_t)threadIdx.x * 16;
-    SeqMap m = seq_identity();
+    if (state->done) return;
+    const uint32_t win = state->win;
+    const uint64_t first = state->pos * kSeqTile;
+    uint32_t es, k_unused;
+    seq_state_split(state->s_bits, &es, &k_unused);
     const float scale = seq_ulp_scale(es < 26u ? 26u : es);
+  for (uint32_t blk = blockIdx.x; blk < win; blk += gridDim.x) {
+    uint64_t base = first + (uint64_t)blk * kSeqTile + (uint64_t)threadIdx.x * 16;
+    SeqMap m = seq_identity();
     if (base + 16 <= n) {
         float4 v[4];
 #pragma unroll
@@ -204,8 +215,41 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
     if (threadIdx.x == 0) {
         SeqMap t = s_wave[0];
         for (int w = 1; w < kBlock / 64; ++w) t = seq_compose(t, s_wave[w]);
-        maps[blockIdx.x] = t;
+        maps[blk] = t;
     }
+    __syncthreads();  // s_wave is rewritten in the next turn
+  }
+}
+
+// Ordered scans of SeqMaps without a barrier per step: inside a wave by shuffles (lane l
+// absorbs what lies to its left), across the waves through one LDS slot per wave.  Returns the
+// composition of everything BEFORE this thread, and in *total the composition of all; NW = waves
+// that carry values (the others pass the identity).  One __syncthreads inside: every thread of
+// the workgroup must call it, and s_w must not be touched again before the next barrier.
+template <int NW>
+__device__ __forceinline__ SeqMap seq_block_before(SeqMap m, SeqMap *s_w, SeqMap *total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int off = 1; off < 64; off <<= 1) {
+        SeqMap o;
+        o.d0 = __shfl_up(m.d0, off);
+        o.d1 = __shfl_up(m.d1, off);
+        if (lane >= off) m = seq_compose(o, m);
+    }
+    if (lane == 63 && wave < NW) s_w[wave] = m;
+    SeqMap ex;  // exclusive inside the wave
+    ex.d0 = __shfl_up(m.d0, 1);
+    ex.d1 = __shfl_up(m.d1, 1);
+    if (lane == 0) ex = seq_identity();
+    __syncthreads();
+    SeqMap pre = seq_identity(), tot = seq_identity();
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        const SeqMap sw = s_w[w];
+        if (w < wave) pre = seq_compose(pre, sw);
+        tot = seq_compose(tot, sw);
+    }
+    *total = tot;
+    return seq_compose(pre, ex);
 }
 
 // One workgroup of 1024 threads ends a window.
@@ -220,51 +264,76 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
 // The new state goes to device memory (for the next window's kernels) and to the pinned
 // host mailbox (the host reads it after synchronising: it sizes the next window).
 __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
-    const SeqMap *__restrict__ maps, const float *__restrict__ x, uint64_t first, uint64_t n,
-    uint32_t nblocks, int use_mask, float thr, SeqState *__restrict__ state,
-    SeqState *__restrict__ host_copy) {
-    __shared__ SeqMap s_a[1024];
-    __shared__ SeqMap s_b[1024];
+    const SeqMap *__restrict__ maps, const float *__restrict__ x, uint64_t n, uint64_t total_blocks,
+    int use_mask, float thr, SeqState *__restrict__ state, SeqState *__restrict__ host_copy) {
+    __shared__ SeqMap s_w[16];
     __shared__ unsigned s_first;
     __shared__ uint32_t s_cross_block, s_cross_k;
     __shared__ uint32_t s_bits_now;
     const uint32_t t = threadIdx.x;
+    if (state->done) return;
+    const uint32_t nblocks = state->win;
+    const uint64_t pos0 = state->pos;
+    const uint64_t first = pos0 * kSeqTile;
+    const uint32_t bits0 = state->s_bits;
     uint32_t es, k0;
-    seq_state_split(state->s_bits, &es, &k0);
+    seq_state_split(bits0, &es, &k0);
+    // ends the window: the state after `advanced` blocks, the next window's size from the
+    // growth of S over this one, mirrored to the host
+    auto finish = [&](uint32_t bits, uint32_t advanced) {
+        const uint64_t pos = pos0 + advanced;
+        const bool finite = ((bits >> 23) & 0xffu) != 0xffu;
+        const double s_before = (double)__uint_as_float(bits0), s_after = (double)__uint_as_float(bits);
+        const double rate = advanced ? (s_after - s_before) / (double)advanced : 0.0;
+        SeqState next;
+        next.s_bits = bits;
+        next.pos = pos;
+        next.error = (advanced == 0 || advanced > nblocks) ? 1u : 0u;
+        next.done = (pos >= total_blocks || !finite || next.error) ? 1u : 0u;
+        next.win = next.done ? 0u : (uint32_t)seq_next_window(pos, total_blocks, s_after, rate);
+        next.saw_nan = 0;
+        next.pad = 0;
+        *state = next;
+        *host_copy = next;
+    };
 
     // ---- (1) scan -----------------------------------------------------------------------
     {
         const uint32_t chunk = (nblocks + 1023u) / 1024u;
         const uint32_t lo = t * chunk;
         const uint32_t hi = lo + chunk < nblocks ? lo + chunk : nblocks;
+        // batches of eight loads in flight (a dependent loop would pay one round trip per map)
         SeqMap mine = seq_identity();
-        for (uint32_t b = lo; b < hi; ++b) mine = seq_compose(mine, maps[b]);
-        if (t == 0) s_first = 0xffffffffu;
-        s_a[t] = mine;
-        __syncthreads();
-        // inclusive Hillis-Steele scan of the per-thread maps (order preserved)
-        SeqMap *src = s_a, *dst = s_b;
-        for (uint32_t off = 1; off < 1024u; off <<= 1) {
-            SeqMap v = src[t];
-            if (t >= off) v = seq_compose(src[t - off], v);
-            dst[t] = v;
-            __syncthreads();
-            SeqMap *tmp = src;
-            src = dst;
-            dst = tmp;
+        for (uint32_t b0 = lo; b0 < hi; b0 += 8) {
+            SeqMap mm[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) mm[i] = maps[b0 + i < hi ? b0 + i : hi - 1];
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (b0 + i < hi) mine = seq_compose(mine, mm[i]);
         }
-        SeqMap before = t == 0 ? seq_identity() : src[t - 1];
+        if (t == 0) s_first = 0xffffffffu;
+        SeqMap all;
+        const SeqMap before = seq_block_before<16>(mine, s_w, &all);
         uint32_t k = seq_apply(before, k0);
         uint32_t cand = 0xffffffffu, cand_k = 0;
         if (k < SEQ_K_LIMIT) {
-            for (uint32_t b = lo; b < hi; ++b) {
-                uint32_t k2 = seq_apply(maps[b], k);
-                if (k2 >= SEQ_K_LIMIT) {
-                    cand = b;
-                    cand_k = k;
-                    break;
+            for (uint32_t b0 = lo; b0 < hi && cand == 0xffffffffu; b0 += 8) {
+                SeqMap mm[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) mm[i] = maps[b0 + i < hi ? b0 + i : hi - 1];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (b0 + i < hi && cand == 0xffffffffu) {
+                        const uint32_t k2 = seq_apply(mm[i], k);
+                        if (k2 >= SEQ_K_LIMIT) {
+                            cand = b0 + i;
+                            cand_k = k;
+                        } else {
+                            k = k2;
+                        }
+                    }
                 }
-                k = k2;
             }
         }
         if (cand != 0xffffffffu) atomicMin(&s_first, cand);
@@ -285,13 +354,7 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     const uint32_t cb = s_cross_block;
     uint32_t k_cur = s_cross_k;
     if (cb == 0xffffffffu) {
-        if (t == 0) {
-            const uint32_t bits = seq_state_join(es, k_cur);
-            state->s_bits = bits;
-            state->next_rel = nblocks;
-            host_copy->s_bits = bits;
-            host_copy->next_rel = nblocks;
-        }
+        if (t == 0) finish(seq_state_join(es, k_cur), nblocks);
         return;
     }
 
@@ -338,28 +401,15 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
                 if (take[i]) m = seq_append_abs(m, a[i], es, scale);
         }
         if (t == 0) s_first = 0xffffffffu;
-        if (holds) s_a[t] = m;
-        __syncthreads();
-        SeqMap *src = s_a, *dst = s_b;
-        for (uint32_t off = 1; off < (uint32_t)kBlock; off <<= 1) {
-            if (holds) {
-                SeqMap v = src[t];
-                if (t >= off) v = seq_compose(src[t - off], v);
-                dst[t] = v;
-            }
-            __syncthreads();
-            SeqMap *tmp = src;
-            src = dst;
-            dst = tmp;
-        }
+        SeqMap all;
+        const SeqMap before = seq_block_before<kBlock / 64>(m, s_w, &all);
         uint32_t k = 0;
         if (holds) {
-            const SeqMap before = t == 0 ? seq_identity() : src[t - 1];
             k = seq_apply(before, k_cur);
             const bool crosses = t >= done && k < SEQ_K_LIMIT && seq_apply(m, k) >= SEQ_K_LIMIT;
             if (crosses) atomicMin(&s_first, t);
         }
-        const uint32_t k_end = seq_apply(src[kBlock - 1], k_cur);  // state after the block if no crossing
+        const uint32_t k_end = seq_apply(all, k_cur);  // state after the block if no crossing
         __syncthreads();
         const uint32_t tstar = s_first;
         if (tstar == 0xffffffffu) {
@@ -391,12 +441,7 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         seq_state_split(result_bits, &es, &k_cur);
         __syncthreads();  // s_first / s_bits_now are rewritten in the next turn
     }
-    if (t == 0) {
-        state->s_bits = result_bits;
-        state->next_rel = cb + 1;
-        host_copy->s_bits = result_bits;
-        host_copy->next_rel = cb + 1;
-    }
+    if (t == 0) finish(result_bits, cb + 1);
 }
 
 __global__ __launch_bounds__(kBlock) void any_nan_kernel(const float *__restrict__ x,
@@ -506,35 +551,38 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     SeqMap *maps = (SeqMap *)((char *)ws + kScratchHeader);
     SeqState *h_state = (SeqState *)ctx->mailbox;
     memset(h_state, 0, sizeof(SeqState));
+    h_state->win = (uint32_t)seq_next_window(0, total_blocks, 0.0, 0.0);
     RBN_HIP(hipMemcpyAsync(&scr->seq, h_state, sizeof(SeqState), hipMemcpyHostToDevice,
                            ctx->stream));
-    uint64_t pos = 0;  // in blocks of kSeqTile elements
-    uint32_t s_bits = 0;
-    double rate = 0.0;  // growth of S per block over the last window
-    while (pos < total_blocks) {
-        if (!is_finite_bits(s_bits)) break;
-        uint32_t es, k;
-        seq_state_split(s_bits, &es, &k);
-        float s_before;
-        memcpy(&s_before, &s_bits, 4);
-        const uint64_t win = seq_next_window(pos, total_blocks, (double)s_before, rate);
-        const uint64_t first = pos * kSeqTile;
-        seq_block_maps_kernel<<<dim3((unsigned)win), dim3(kBlock), 0, ctx->stream>>>(
-            d_x, first, n, es, use_mask, thr, maps);
-        // ends the window; also writes the new state to the pinned mailbox
-        seq_scan_replay_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(
-            maps, d_x, first, n, (uint32_t)win, use_mask, thr, &scr->seq, h_state);
+    // Windows are queued in batches: the kernels take each window from the device state and
+    // return at once when the sum is complete, so the host only looks in between batches and
+    // sizes the next one by the binades S still has to climb (a window ends where S leaves
+    // its binade).
+    const unsigned grid = (unsigned)(total_blocks < 8192 ? total_blocks : 8192);
+    int batch = 4;
+    for (;;) {
+        for (int i = 0; i < batch; ++i) {
+            seq_block_maps_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(d_x, n, use_mask, thr,
+                                                                               &scr->seq, maps);
+            seq_scan_replay_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(
+                maps, d_x, n, total_blocks, use_mask, thr, &scr->seq, h_state);
+        }
         RBN_HIP(hipGetLastError());
         RBN_HIP(hipStreamSynchronize(ctx->stream));
-        s_bits = h_state->s_bits;
-        const uint32_t advanced = h_state->next_rel;
-        if (advanced == 0 || advanced > win)
+        if (h_state->error)
             return rbn_fail(RBN_ERR_HIP, "sequential-sum scan made no progress (internal error)");
-        float s_after;
-        memcpy(&s_after, &s_bits, 4);
-        rate = ((double)s_after - (double)s_before) / (double)advanced;
-        pos += advanced;
+        if (h_state->done) break;
+        float s_now;
+        memcpy(&s_now, &h_state->s_bits, 4);
+        // S grows by about s_now * (blocks left / blocks done) more: one window per doubling
+        const double done_blocks = (double)h_state->pos, left = (double)(total_blocks - h_state->pos);
+        const double growth = 1.0 + left / (done_blocks > 1.0 ? done_blocks : 1.0);
+        batch = (int)(log2(growth) + 1.5);
+        batch = batch < 1 ? 1 : (batch > 16 ? 16 : batch);
+        (void)s_now;
     }
+    const uint32_t s_bits = h_state->s_bits;
+    const uint64_t pos = h_state->pos;
     float s;
     memcpy(&s, &s_bits, 4);
     if (!is_finite_bits(s_bits) && s == s && pos < total_blocks && !use_mask) {

@@ -94,6 +94,61 @@ __global__ __launch_bounds__(kBlock) void act_quant_i8_kernel(
     }
 }
 
+// The same with the row kept in registers between the two passes (NQ 16-byte pieces per
+// thread, K <= 1024 * NQ, K % 4 == 0, 16-byte aligned rows): the row is read from memory once,
+// with all its loads in flight before the first comparison.
+template <int NQ>
+__global__ __launch_bounds__(kBlock) void act_quant_i8_regs_kernel(
+    const float *__restrict__ x, uint64_t K, uint64_t pitch, int8_t *__restrict__ q,
+    float *__restrict__ act_scale, int32_t *__restrict__ rowsum) {
+    __shared__ float s_max[kBlock / 64];
+    __shared__ int s_sum[kBlock / 64];
+    const uint64_t m = blockIdx.x;
+    const float4 *row = reinterpret_cast<const float4 *>(x + m * K);
+    const uint32_t quads = (uint32_t)(K / 4), out_quads = (uint32_t)(pitch / 4);
+    float4 v[NQ];
+#pragma unroll
+    for (int j = 0; j < NQ; ++j) {
+        const uint32_t qd = threadIdx.x + j * kBlock;
+        v[j] = row[qd < quads ? qd : quads - 1];
+    }
+    float amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NQ; ++j) {
+        const uint32_t qd = threadIdx.x + j * kBlock;
+        if (qd >= quads) v[j] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);  // the zero padding
+        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(v[j].x), fabsf(v[j].y)), fmaxf(fabsf(v[j].z), fabsf(v[j].w))));
+    }
+    amax = wave_max(amax);
+    if ((threadIdx.x & 63) == 0) s_max[threadIdx.x >> 6] = amax;
+    __syncthreads();
+    amax = s_max[0];
+    for (int w = 1; w < kBlock / 64; ++w) amax = fmaxf(amax, s_max[w]);
+    const float g = fmaxf(amax, 1e-5f);
+    const float inv = 127.0f / g;
+    int sum = 0;
+    uint32_t *qrow = reinterpret_cast<uint32_t *>(q + m * pitch);
+#pragma unroll
+    for (int j = 0; j < NQ; ++j) {
+        const uint32_t qd = threadIdx.x + j * kBlock;
+        const int a = quant1(v[j].x, inv), b = quant1(v[j].y, inv), c = quant1(v[j].z, inv),
+                  d = quant1(v[j].w, inv);
+        sum += a + b + c + d;
+        if (qd < out_quads)
+            qrow[qd] = (uint32_t)(a & 0xff) | ((uint32_t)(b & 0xff) << 8) | ((uint32_t)(c & 0xff) << 16) |
+                       ((uint32_t)(d & 0xff) << 24);
+    }
+    sum = wave_sum(sum);
+    if ((threadIdx.x & 63) == 0) s_sum[threadIdx.x >> 6] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int t = 0;
+        for (int w = 0; w < kBlock / 64; ++w) t += s_sum[w];
+        rowsum[m] = t;
+        act_scale[m] = g / 127.0f;
+    }
+}
+
 __global__ void fill_f32_kernel(float *dst, float value, uint64_t n) {
     uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) dst[i] = value;
@@ -111,8 +166,20 @@ int rbn_act_quant_i8(rbn_ctx *ctx, const float *d_x, uint64_t M, uint64_t K, int
     RBN_REQUIRE(((uintptr_t)d_x & 3u) == 0 && ((uintptr_t)d_q & 15u) == 0,
                 "d_x must be 4-byte and d_q 16-byte aligned");
     RBN_REQUIRE(M <= 0x7fffffffull, "too many rows");
-    act_quant_i8_kernel<<<dim3((unsigned)M), dim3(kBlock), 0, ctx->stream>>>(
-        d_x, K, rbn_kpad(K), d_q, d_act_scale, d_rowsum);
+    const uint64_t pitch = rbn_kpad(K);
+    const bool in_regs = (K & 3) == 0 && ((uintptr_t)d_x & 15u) == 0 && pitch <= 16ull * 4 * kBlock;
+    if (in_regs && pitch <= 4ull * 4 * kBlock)
+        act_quant_i8_regs_kernel<4><<<dim3((unsigned)M), dim3(kBlock), 0, ctx->stream>>>(
+            d_x, K, pitch, d_q, d_act_scale, d_rowsum);
+    else if (in_regs && pitch <= 8ull * 4 * kBlock)
+        act_quant_i8_regs_kernel<8><<<dim3((unsigned)M), dim3(kBlock), 0, ctx->stream>>>(
+            d_x, K, pitch, d_q, d_act_scale, d_rowsum);
+    else if (in_regs)
+        act_quant_i8_regs_kernel<16><<<dim3((unsigned)M), dim3(kBlock), 0, ctx->stream>>>(
+            d_x, K, pitch, d_q, d_act_scale, d_rowsum);
+    else
+        act_quant_i8_kernel<<<dim3((unsigned)M), dim3(kBlock), 0, ctx->stream>>>(
+            d_x, K, pitch, d_q, d_act_scale, d_rowsum);
     RBN_HIP(hipGetLastError());
     return RBN_OK;
 }

@@ -195,8 +195,11 @@ def test_tile_weights_sanitises_invalid_code(ctx):
 
 # ---- (2) activation quantisation -----------------------------------------------------------
 
-@pytest.mark.parametrize("M,K", [(1, 2048), (1, 4096), (4, 11008), (16, 4096), (3, 100), (5, 1), (2, 67)])
+@pytest.mark.parametrize("M,K", [(1, 2048), (1, 4096), (4, 11008), (16, 4096), (3, 100), (5, 1), (2, 67),
+                                 (3, 4100), (5, 8192), (4, 16384), (3, 16388), (2, 20000), (300, 1028)])
 def test_act_quant_i8(ctx, M, K):
+    # K % 4 == 0 up to 16384: the row stays in registers (4, 8 or 16 pieces per thread);
+    # other K, or longer rows: two passes over the row
     x = synth_normal(0x5EED0001, 1.0, (M, K))
     if M >= 3:
         x[1, :] = 0.0                  # zero token: guarded scale, all zeros

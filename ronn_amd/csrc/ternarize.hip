@@ -29,8 +29,10 @@ __device__ __forceinline__ uint32_t ternary_code(float v, float threshold) {
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(kBlock) void pack_ternary_kernel(
     const float *__restrict__ x, uint64_t n, float threshold, uint32_t *__restrict__ packed,
-    uint64_t n_tiles, unsigned long long *__restrict__ survivors) {
+    uint64_t n_tiles, unsigned long long *__restrict__ survivors, double *__restrict__ psum) {
     __shared__ unsigned s_cnt[kBlock / 64];
+    __shared__ double s_sum[kBlock / 64];
+    double acc = 0.0;  // sum of the survivors' |x| (tree mode: one partial per workgroup)
     const uint64_t n_quads = (n + 3) / 4;
     const uint64_t n_words = (n + 15) / 16;
     unsigned count = 0;
@@ -54,7 +56,9 @@ __global__ __launch_bounds__(kBlock) void pack_ternary_kernel(
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     byte |= ternary_code(e[i], threshold) << (2 * i);
-                    count += fabsf(e[i]) > threshold ? 1u : 0u;
+                    const bool keep = fabsf(e[i]) > threshold;
+                    count += keep ? 1u : 0u;
+                    if (psum) acc += keep ? (double)fabsf(e[i]) : 0.0;
                 }
             } else if (q < n_quads) {  // the single partial group at the tail
                 for (int i = 0; i < 4; ++i) {
@@ -62,7 +66,9 @@ __global__ __launch_bounds__(kBlock) void pack_ternary_kernel(
                     if (idx < n) {
                         float e = x[idx];
                         byte |= ternary_code(e, threshold) << (2 * i);
-                        count += fabsf(e) > threshold ? 1u : 0u;
+                        const bool keep = fabsf(e) > threshold;
+                        count += keep ? 1u : 0u;
+                        if (psum) acc += keep ? (double)fabsf(e) : 0.0;
                     }
                 }
             }
@@ -84,6 +90,32 @@ __global__ __launch_bounds__(kBlock) void pack_ternary_kernel(
             if (t) atomicAdd(survivors, t);
         }
     }
+    if (psum) {
+        // fixed order: lanes by shuffles, waves in turn, workgroups by the final kernel
+        for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off);
+        if ((threadIdx.x & 63) == 0) s_sum[threadIdx.x >> 6] = acc;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            double t = 0.0;
+            for (int w = 0; w < kBlock / 64; ++w) t += s_sum[w];
+            psum[blockIdx.x] = t;
+        }
+    }
+}
+
+// Sum of the per-workgroup partials of the kernel above, in a fixed order.
+__global__ __launch_bounds__(kBlock) void sum_partials_kernel(const double *__restrict__ psum,
+                                                             int nparts, float *__restrict__ out) {
+    __shared__ double s_sum[kBlock];
+    double acc = 0.0;
+    for (int i = threadIdx.x; i < nparts; i += kBlock) acc += psum[i];
+    s_sum[threadIdx.x] = acc;
+    __syncthreads();
+    for (int off = kBlock / 2; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) s_sum[threadIdx.x] += s_sum[threadIdx.x + off];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *out = (float)s_sum[0];
 }
 
 // ---------------------------------------------------------------------------
@@ -96,15 +128,35 @@ __global__ __launch_bounds__(kBlock) void abs_sum_tree_partial_kernel(
     __shared__ unsigned long long s_cnt[kBlock];
     double acc = 0.0;
     unsigned long long cnt = 0;
-    uint64_t stride = (uint64_t)gridDim.x * kBlock;
-    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += stride) {
-        float a = fabsf(x[i]);
-        bool take = use_mask ? (a > thr) : true;
-        if (take) {
-            acc += (double)a;
-            ++cnt;
+    const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+    const uint64_t tid = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    auto add = [&](float v) {
+        const float a = fabsf(v);
+        const bool take = use_mask ? (a > thr) : true;
+        acc += take ? (double)a : 0.0;
+        cnt += take ? 1u : 0u;
+    };
+    // 16-byte loads, four in flight per thread; a scalar loop for what is left (or for an
+    // unaligned tensor).  The order of the additions is fixed by the grid, hence deterministic.
+    uint64_t done = 0;
+    if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0) {
+        const float4 *x4 = reinterpret_cast<const float4 *>(x);
+        const uint64_t n4 = n / 4;
+        uint64_t i = tid;
+        for (; i + 3 * stride < n4; i += 4 * stride) {
+            const float4 a = x4[i], b = x4[i + stride], c = x4[i + 2 * stride], d = x4[i + 3 * stride];
+            add(a.x), add(a.y), add(a.z), add(a.w);
+            add(b.x), add(b.y), add(b.z), add(b.w);
+            add(c.x), add(c.y), add(c.z), add(c.w);
+            add(d.x), add(d.y), add(d.z), add(d.w);
         }
+        for (; i < n4; i += stride) {
+            const float4 a = x4[i];
+            add(a.x), add(a.y), add(a.z), add(a.w);
+        }
+        done = n4 * 4;
     }
+    for (uint64_t i = done + tid; i < n; i += stride) add(x[i]);
     s_sum[threadIdx.x] = acc;
     s_cnt[threadIdx.x] = cnt;
     __syncthreads();
@@ -627,31 +679,44 @@ int tree_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, float
     return RBN_OK;
 }
 
-// pack + survivor count (count returned through the mailbox when h_survivors != NULL)
+// pack + survivor count (count returned through the mailbox when h_survivors != NULL) and,
+// when h_survivor_sum != NULL, the survivors' sum of |x| as a deterministic f64 tree (the
+// tree mode's scale rides on the packing pass; the strict mode's cannot)
+constexpr int kPackGrid = 8192;
 int pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold, uint8_t *d_packed,
-                 uint64_t *h_survivors) {
+                 uint64_t *h_survivors, float *h_survivor_sum = nullptr) {
     if (n == 0) {
         if (h_survivors) *h_survivors = 0;
+        if (h_survivor_sum) *h_survivor_sum = -0.0f;
         return RBN_OK;
     }
     unsigned long long *d_cnt = nullptr;
-    if (h_survivors) {
+    double *d_psum = nullptr;
+    ReduceScratch *scr = nullptr;
+    if (h_survivors || h_survivor_sum) {
         void *ws = nullptr;
-        RBN_CHECK(rbn_workspace(ctx, kScratchHeader, &ws));
-        d_cnt = &((ReduceScratch *)ws)->survivors;
+        RBN_CHECK(rbn_workspace(ctx, kScratchHeader + (size_t)kPackGrid * sizeof(double), &ws));
+        scr = (ReduceScratch *)ws;
+        d_cnt = &scr->survivors;
+        if (h_survivor_sum) d_psum = (double *)((char *)ws + kScratchHeader);
         memset(ctx->mailbox, 0, 8);
         RBN_HIP(hipMemcpyAsync(d_cnt, ctx->mailbox, 8, hipMemcpyHostToDevice, ctx->stream));
     }
     uint64_t tiles = (n + kSeqTile - 1) / kSeqTile;
     if (tiles > 0x7fffffffull) return rbn_fail(RBN_ERR_UNSUPPORTED, "tensor too large");
-    const unsigned grid = (unsigned)(tiles < 8192 ? tiles : 8192);
+    const unsigned grid = (unsigned)(tiles < (uint64_t)kPackGrid ? tiles : (uint64_t)kPackGrid);
     pack_ternary_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
-        d_x, n, threshold, (uint32_t *)d_packed, tiles, d_cnt);
+        d_x, n, threshold, (uint32_t *)d_packed, tiles, d_cnt, d_psum);
+    if (d_psum)
+        sum_partials_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(d_psum, (int)grid, &scr->tree_sum);
     RBN_HIP(hipGetLastError());
-    if (h_survivors) {
-        RBN_HIP(hipMemcpyAsync(ctx->mailbox, d_cnt, 8, hipMemcpyDeviceToHost, ctx->stream));
+    if (scr) {
+        char *mb = (char *)ctx->mailbox;
+        RBN_HIP(hipMemcpyAsync(mb, d_cnt, 8, hipMemcpyDeviceToHost, ctx->stream));
+        if (d_psum) RBN_HIP(hipMemcpyAsync(mb + 8, &scr->tree_sum, 4, hipMemcpyDeviceToHost, ctx->stream));
         RBN_HIP(hipStreamSynchronize(ctx->stream));
-        memcpy(h_survivors, ctx->mailbox, 8);
+        if (h_survivors) memcpy(h_survivors, mb, 8);
+        if (h_survivor_sum) memcpy(h_survivor_sum, mb + 8, 4);
     }
     return RBN_OK;
 }
@@ -714,15 +779,13 @@ int rbn_quantize_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, int mode, u
     volatile float threshold = mean * 0.7f;
     // quantization.rs:100 (pack) and the survivor count of :82-91
     uint64_t survivors = 0;
-    RBN_CHECK(pack_ternary(ctx, d_x, n, threshold, d_packed, &survivors));
+    float nz_sum = 0.0f;
+    RBN_CHECK(pack_ternary(ctx, d_x, n, threshold, d_packed, &survivors,
+                           mode == RBN_SUM_TREE ? &nz_sum : nullptr));
     // quantization.rs:93-97
     float scale = 1.0f;
     if (survivors != 0) {
-        float nz_sum = 0.0f;
-        if (mode == RBN_SUM_TREE)
-            RBN_CHECK(tree_abs_sum(ctx, d_x, n, 1, threshold, &nz_sum, nullptr));
-        else
-            RBN_CHECK(strict_abs_sum(ctx, d_x, n, 1, threshold, &nz_sum));
+        if (mode != RBN_SUM_TREE) RBN_CHECK(strict_abs_sum(ctx, d_x, n, 1, threshold, &nz_sum));
         volatile float sc = nz_sum / (float)survivors;
         scale = sc;
     }

@@ -214,16 +214,25 @@ struct SeqState {
     uint32_t error;     // a window made no progress (internal error)
     uint32_t saw_nan;   // set by any_nan_kernel
     uint32_t pad;
+    uint64_t fresh_from;  // blocks from here on have not been seen by any window yet
 };
 
 // One SeqMap per block of 4096 elements, valid for a state of biased exponent `es`.
 // The window and the exponent come from the state; the grid strides over the window's blocks.
+// With `packed` given (masked sums only: thr is the ternary threshold) the kernel also packs
+// every block that no earlier window has touched - a thread's 16 elements are one 32-bit word
+// of the reference's layout - and adds their survivors to this workgroup's counter: the
+// scale's sum and the packing then share one pass over the tensor.
 __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
     const float *__restrict__ x, uint64_t n, int use_mask, float thr,
-    const SeqState *__restrict__ state, SeqMap *__restrict__ maps) {
+    const SeqState *__restrict__ state, SeqMap *__restrict__ maps, uint32_t *__restrict__ packed,
+    unsigned long long *__restrict__ count_parts) {
     __shared__ SeqMap s_wave[kBlock / 64];
+    __shared__ unsigned s_cnt[kBlock / 64];
     if (state->done) return;
     const uint32_t win = state->win;
+    const uint64_t fresh_from = state->fresh_from, pos = state->pos;
+    unsigned fresh_count = 0;
     const uint64_t first = state->pos * kSeqTile;
     uint32_t es, k_unused;
     seq_state_split(state->s_bits, &es, &k_unused);
@@ -231,6 +240,8 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
   for (uint32_t blk = blockIdx.x; blk < win; blk += gridDim.x) {
     uint64_t base = first + (uint64_t)blk * kSeqTile + (uint64_t)threadIdx.x * 16;
     SeqMap m = seq_identity();
+    const bool fresh = packed != nullptr && pos + blk >= fresh_from;
+    uint32_t word = 0;
     if (base + 16 <= n) {
         float4 v[4];
 #pragma unroll
@@ -243,17 +254,28 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
                 float a = fabsf(e[i]);
                 bool take = use_mask ? (a > thr) : true;
                 if (take) m = seq_append_abs(m, a, es, scale);
+                if (fresh) {
+                    word |= ternary_code(e[i], thr) << (2 * (4 * j + i));
+                    fresh_count += take ? 1u : 0u;
+                }
             }
         }
+        if (fresh) packed[base >> 4] = word;
     } else {
         for (int i = 0; i < 16; ++i) {
             uint64_t idx = base + i;
             if (idx < n) {
-                float a = fabsf(x[idx]);
+                float e = x[idx];
+                float a = fabsf(e);
                 bool take = use_mask ? (a > thr) : true;
                 if (take) m = seq_append_abs(m, a, es, scale);
+                if (fresh) {
+                    word |= ternary_code(e, thr) << (2 * i);
+                    fresh_count += take ? 1u : 0u;
+                }
             }
         }
+        if (fresh && base < n) packed[base >> 4] = word;  // tail bits stay zero
     }
     // ordered tree over the wave: lane l absorbs lane l+off (its right neighbour)
     for (int off = 1; off < 64; off <<= 1) {
@@ -271,6 +293,35 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
     }
     __syncthreads();  // s_wave is rewritten in the next turn
   }
+    if (packed) {
+        // one plain read-modify-write per workgroup and launch: slot blockIdx.x belongs to
+        // this workgroup alone, and launches are ordered by the stream
+        for (int off = 32; off > 0; off >>= 1) fresh_count += __shfl_down(fresh_count, off);
+        if ((threadIdx.x & 63) == 0) s_cnt[threadIdx.x >> 6] = fresh_count;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            unsigned t = 0;
+            for (int w = 0; w < kBlock / 64; ++w) t += s_cnt[w];
+            if (t) count_parts[blockIdx.x] += t;
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void fill_u64_kernel(unsigned long long *p, int n) {
+    for (int i = threadIdx.x; i < n; i += kBlock) p[i] = 0;
+}
+__global__ __launch_bounds__(kBlock) void sum_u64_kernel(const unsigned long long *__restrict__ p, int n,
+                                                        unsigned long long *__restrict__ out) {
+    __shared__ unsigned long long s[kBlock];
+    unsigned long long acc = 0;
+    for (int i = threadIdx.x; i < n; i += kBlock) acc += p[i];
+    s[threadIdx.x] = acc;
+    __syncthreads();
+    for (int off = kBlock / 2; off > 0; off >>= 1) {
+        if ((int)threadIdx.x < off) s[threadIdx.x] += s[threadIdx.x + off];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) *out = s[0];
 }
 
 // Ordered scans of SeqMaps without a barrier per step: inside a wave by shuffles (lane l
@@ -345,6 +396,8 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         next.win = next.done ? 0u : (uint32_t)seq_next_window(pos, total_blocks, s_after, rate);
         next.saw_nan = 0;
         next.pad = 0;
+        const uint64_t seen = pos0 + nblocks, before = state->fresh_from;
+        next.fresh_from = seen > before ? seen : before;
         *state = next;
         *host_copy = next;
     };
@@ -590,17 +643,27 @@ constexpr int kTreeParts = 2048;
 inline bool is_finite_bits(uint32_t b) { return ((b >> 23) & 0xffu) != 0xffu; }
 
 // Exact sequential sum (optionally masked) of |x| over n elements.
+int pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold, uint8_t *d_packed,
+                 uint64_t *h_survivors, float *h_survivor_sum);
+
+// With d_packed given (use_mask must be set, thr is the ternary threshold) the same pass also
+// packs the tensor and counts the survivors into *h_survivors.
 int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, float thr,
-                   float *h_sum) {
+                   float *h_sum, uint8_t *d_packed = nullptr, uint64_t *h_survivors = nullptr) {
     if (n == 0) {
         *h_sum = -0.0f;  // Rust's empty f32 sum
+        if (h_survivors) *h_survivors = 0;
         return RBN_OK;
     }
+    constexpr int kMapGrid = 8192;
     const uint64_t total_blocks = (n + kSeqTile - 1) / kSeqTile;
     void *ws = nullptr;
-    RBN_CHECK(rbn_workspace(ctx, kScratchHeader + total_blocks * sizeof(SeqMap), &ws));
+    RBN_CHECK(rbn_workspace(ctx, kScratchHeader + total_blocks * sizeof(SeqMap) + kMapGrid * 8, &ws));
     ReduceScratch *scr = (ReduceScratch *)ws;
     SeqMap *maps = (SeqMap *)((char *)ws + kScratchHeader);
+    unsigned long long *count_parts =
+        d_packed ? (unsigned long long *)((char *)ws + kScratchHeader + total_blocks * sizeof(SeqMap)) : nullptr;
+    if (d_packed) fill_u64_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(count_parts, kMapGrid);
     SeqState *h_state = (SeqState *)ctx->mailbox;
     memset(h_state, 0, sizeof(SeqState));
     h_state->win = (uint32_t)seq_next_window(0, total_blocks, 0.0, 0.0);
@@ -610,12 +673,12 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     // return at once when the sum is complete, so the host only looks in between batches and
     // sizes the next one by the binades S still has to climb (a window ends where S leaves
     // its binade).
-    const unsigned grid = (unsigned)(total_blocks < 8192 ? total_blocks : 8192);
+    const unsigned grid = (unsigned)(total_blocks < (uint64_t)kMapGrid ? total_blocks : (uint64_t)kMapGrid);
     int batch = 4;
     for (;;) {
         for (int i = 0; i < batch; ++i) {
-            seq_block_maps_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(d_x, n, use_mask, thr,
-                                                                               &scr->seq, maps);
+            seq_block_maps_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
+                d_x, n, use_mask, thr, &scr->seq, maps, (uint32_t *)d_packed, count_parts);
             seq_scan_replay_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(
                 maps, d_x, n, total_blocks, use_mask, thr, &scr->seq, h_state);
         }
@@ -648,6 +711,19 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
         if (h_state->saw_nan) s = NAN;
     }
     *h_sum = s;
+    if (d_packed) {
+        if (pos < total_blocks) {
+            // the sum left the finite range before the end: the windows stopped there, so
+            // pack (and count) with the plain kernel
+            RBN_CHECK(pack_ternary(ctx, d_x, n, thr, d_packed, h_survivors, nullptr));
+        } else {
+            sum_u64_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(count_parts, (int)grid, &scr->survivors);
+            RBN_HIP(hipGetLastError());
+            RBN_HIP(hipMemcpyAsync(ctx->mailbox, &scr->survivors, 8, hipMemcpyDeviceToHost, ctx->stream));
+            RBN_HIP(hipStreamSynchronize(ctx->stream));
+            if (h_survivors) memcpy(h_survivors, ctx->mailbox, 8);
+        }
+    }
     return RBN_OK;
 }
 
@@ -684,7 +760,7 @@ int tree_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, float
 // tree mode's scale rides on the packing pass; the strict mode's cannot)
 constexpr int kPackGrid = 8192;
 int pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold, uint8_t *d_packed,
-                 uint64_t *h_survivors, float *h_survivor_sum = nullptr) {
+                 uint64_t *h_survivors, float *h_survivor_sum) {
     if (n == 0) {
         if (h_survivors) *h_survivors = 0;
         if (h_survivor_sum) *h_survivor_sum = -0.0f;
@@ -756,7 +832,7 @@ int rbn_pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold
     if (n == 0) return RBN_OK;
     RBN_CHECK(check_f32_ptr(d_x, "d_x"));
     RBN_REQUIRE(d_packed && ((uintptr_t)d_packed & 3u) == 0, "d_packed must be 4-byte aligned");
-    return pack_ternary(ctx, d_x, n, threshold, d_packed, nullptr);
+    return pack_ternary(ctx, d_x, n, threshold, d_packed, nullptr, nullptr);
 }
 
 int rbn_quantize_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, int mode, uint8_t *d_packed,
@@ -778,14 +854,16 @@ int rbn_quantize_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, int mode, u
     volatile float mean = sum / (float)n;
     volatile float threshold = mean * 0.7f;
     // quantization.rs:100 (pack) and the survivor count of :82-91
+    // (one pass in either mode: the survivors' sum, their count and the packed words)
     uint64_t survivors = 0;
     float nz_sum = 0.0f;
-    RBN_CHECK(pack_ternary(ctx, d_x, n, threshold, d_packed, &survivors,
-                           mode == RBN_SUM_TREE ? &nz_sum : nullptr));
+    if (mode == RBN_SUM_TREE)
+        RBN_CHECK(pack_ternary(ctx, d_x, n, threshold, d_packed, &survivors, &nz_sum));
+    else
+        RBN_CHECK(strict_abs_sum(ctx, d_x, n, 1, threshold, &nz_sum, d_packed, &survivors));
     // quantization.rs:93-97
     float scale = 1.0f;
     if (survivors != 0) {
-        if (mode != RBN_SUM_TREE) RBN_CHECK(strict_abs_sum(ctx, d_x, n, 1, threshold, &nz_sum));
         volatile float sc = nz_sum / (float)survivors;
         scale = sc;
     }

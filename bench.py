@@ -2,7 +2,7 @@
 """Benchmark of the BitNet ternary hot path on one MI355X.
 
 Headline (the JSON line's `value`): decode-regime ternary GEMV at K=4096, N=11008,
-M=1 (the FFN up/gate shape of BASELINE.json's decode sweep), int8 activations and
+M=1 (the FFN up/gate shape of the decode sweep), int8 activations and
 tiled 2-bit weights already resident in HBM.  One step = one GEMV launch.  The steps
 rotate over enough distinct weight buffers (> 256 MiB in total) that every launch
 streams its weights from HBM rather than from the Infinity Cache; launches are

@@ -291,7 +291,7 @@ def test_gemv_decode_sweep_shapes(ctx, M, K, N):
 
 
 def test_gemv_reference_mode_config1(ctx):
-    # BASELINE config 1: x[1,2048] . W[2048,2048], both operands ternarised as the reference does
+    # the single-BitLinear configuration, x[1,2048] . W[2048,2048], both operands ternarised as the reference does
     x = synth_normal(0x5EED0001, 1.0, (1, 2048))
     w = synth_normal(0x5EED1001, 0.02, (2048, 2048))
     want_out, want_acc = O.execute_ternary(x, w)

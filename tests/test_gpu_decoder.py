@@ -24,7 +24,8 @@ def close(a, b, rtol=1e-4, atol=1e-5):
     return np.allclose(a, b, rtol=rtol, atol=atol)
 
 
-@pytest.mark.parametrize("M,H", [(1, 2560), (5, 256), (3, 6912), (2, 100), (4, 8192)])
+@pytest.mark.parametrize("M,H", [(1, 2560), (5, 256), (3, 6912), (2, 100), (4, 8192),
+                                 (64, 2560), (9, 8192), (33, 100), (12, 6912), (8, 102)])
 @pytest.mark.parametrize("with_delta", [False, True])
 def test_rmsnorm_quant(ctx, M, H, with_delta):
     x = synth_normal(11 + M, 1.0, (M, H))
@@ -49,7 +50,7 @@ def test_rmsnorm_quant(ctx, M, H, with_delta):
         assert (d_x.download(np.float32, M * H).reshape(M, H) == xin).all()
 
 
-@pytest.mark.parametrize("M,F", [(1, 6912), (3, 384), (2, 1000)])
+@pytest.mark.parametrize("M,F", [(1, 6912), (3, 384), (2, 1000), (40, 6912), (8, 1000), (16, 8192)])
 def test_rmsnorm_quant_with_swiglu_input(ctx, M, F):
     gu = synth_normal(41 + M, 2.0, (M, 2 * F))
     g = (1.0 + synth_normal(42, 0.1, (F,))).astype(np.float32)

@@ -314,7 +314,16 @@ __global__ __launch_bounds__(kBlock) void sum_u64_kernel(const unsigned long lon
                                                         unsigned long long *__restrict__ out) {
     __shared__ unsigned long long s[kBlock];
     unsigned long long acc = 0;
-    for (int i = threadIdx.x; i < n; i += kBlock) acc += p[i];
+    for (int i0 = 0; i0 < n; i0 += 8 * kBlock) {  // eight loads in flight per thread
+        unsigned long long v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int i = i0 + j * kBlock + (int)threadIdx.x;
+            v[j] = p[i < n ? i : n - 1];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc += (i0 + j * kBlock + (int)threadIdx.x) < n ? v[j] : 0ull;
+    }
     s[threadIdx.x] = acc;
     __syncthreads();
     for (int off = kBlock / 2; off > 0; off >>= 1) {

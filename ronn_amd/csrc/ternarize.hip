@@ -108,7 +108,16 @@ __global__ __launch_bounds__(kBlock) void sum_partials_kernel(const double *__re
                                                              int nparts, float *__restrict__ out) {
     __shared__ double s_sum[kBlock];
     double acc = 0.0;
-    for (int i = threadIdx.x; i < nparts; i += kBlock) acc += psum[i];
+    for (int i0 = 0; i0 < nparts; i0 += 8 * kBlock) {  // eight loads in flight per thread
+        double v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int i = i0 + j * kBlock + (int)threadIdx.x;
+            v[j] = psum[i < nparts ? i : nparts - 1];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc += (i0 + j * kBlock + (int)threadIdx.x) < nparts ? v[j] : 0.0;
+    }
     s_sum[threadIdx.x] = acc;
     __syncthreads();
     for (int off = kBlock / 2; off > 0; off >>= 1) {

@@ -343,13 +343,7 @@ def main():
                                     "note": "single 11 MiB weight buffer re-read from cache, not HBM"}
         del one
         def kernel_for(m, k, n):
-            # the choice rbn_matmul_t2_i8 makes (csrc/gemm_mfma.hip)
-            if m <= 3:
-                return "gemv"
-            kn = k * n
-            if m <= 16 or (m <= 32 and kn < (1 << 27)) or (m <= 64 and kn < (1 << 25)):
-                return "skinny_mfma"
-            return "gemm_mfma"
+            return ("gemv", "skinny_mfma", "gemm_mfma")[ctx.lib.rbn_matmul_kernel_choice(m, k, n)]
 
         def sweep_over(shapes, ms, sigma):
             rows = []

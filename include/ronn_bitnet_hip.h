@@ -206,6 +206,11 @@ int rbn_gemm_t2_i8_mfma(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scal
 int rbn_matmul_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
                      const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
                      uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);
+/* Which of the three kernels rbn_matmul_t2_i8 runs for a shape (needs no device). */
+#define RBN_KERNEL_GEMV 0
+#define RBN_KERNEL_SKINNY 1
+#define RBN_KERNEL_MFMA 2
+int rbn_matmul_kernel_choice(uint64_t M, uint64_t K, uint64_t N);
 
 /* ---- whole execute(): CompiledKernel::execute, TernaryMatMul arm,
  *      kernels.rs:271-283 ---------------------------------------------------- */

@@ -101,6 +101,7 @@ SIGNATURES = {
     "rbn_add_i32": (C.c_int, [_vp, _vp, C.c_int32]),
     "rbn_synth_normal_device_f32": (C.c_int, [_vp, _u64, C.c_float, _vp, _u64]),
     "rbn_probe_mfma_i8": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_double)]),
+    "rbn_matmul_kernel_choice": (C.c_int, [_u64, _u64, _u64]),
     "rbn_matmul_t2_i8": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
     "rbn_execute_ternary_matmul": (C.c_int, [_vp, _vp, _vp, _u64, _u64, _u64, C.c_int, _vp, _vp]),
     "rbn_synth_normal_f32": (None, [_u64, C.c_double, _u64, _u64, _vp]),

@@ -437,22 +437,29 @@ extern "C" int rbn_gemm_t2_i8_mfma(rbn_ctx *ctx, const int8_t *d_q, const float 
     return RBN_OK;
 }
 
+extern "C" int rbn_matmul_kernel_choice(uint64_t M, uint64_t K, uint64_t N) {
+    // measured crossovers: the dot-instruction GEMV wins up to three tokens; the streaming
+    // small-batch kernel up to 32 tokens (16 on very large matrices) and, on small matrices,
+    // up to its limit of 64; the tiled kernel beyond
+    if (M <= 3) return RBN_KERNEL_GEMV;
+    const uint64_t kn = K * N;
+    if (M <= 16 || (M <= 32 && kn < (1ull << 27)) || (M <= RBN_SKINNY_MAX_M && kn < (1ull << 25)))
+        return RBN_KERNEL_SKINNY;
+    return RBN_KERNEL_MFMA;
+}
+
 extern "C" int rbn_matmul_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
                                 const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
                                 uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc,
                                 float *d_out) {
-    // measured crossovers: the dot-instruction GEMV wins up to three tokens; the streaming
-    // small-batch kernel up to 32 tokens (16 on very large matrices) and, on small matrices,
-    // up to its limit of 64; the tiled kernel beyond
-    if (M <= 3)
-        return rbn_gemv_t2_i8(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N, d_acc,
-                              d_out);
-    const uint64_t kn = K * N;
-    const bool skinny = M <= 16 || (M <= 32 && kn < (1ull << 27)) ||
-                        (M <= RBN_SKINNY_MAX_M && kn < (1ull << 25));
-    if (skinny)
-        return rbn_gemm_t2_i8_skinny(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N,
-                                     d_acc, d_out);
-    return rbn_gemm_t2_i8_mfma(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N, d_acc,
-                               d_out);
+    switch (rbn_matmul_kernel_choice(M, K, N)) {
+        case RBN_KERNEL_GEMV:
+            return rbn_gemv_t2_i8(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N, d_acc, d_out);
+        case RBN_KERNEL_SKINNY:
+            return rbn_gemm_t2_i8_skinny(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N, d_acc,
+                                         d_out);
+        default:
+            return rbn_gemm_t2_i8_mfma(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N, d_acc,
+                                       d_out);
+    }
 }

@@ -79,7 +79,8 @@ __global__ __launch_bounds__(W * 64) void bitlinear_gemv_kernel(
     const float *__restrict__ x,        // [K], or gate|up [2K] with SWIGLU
     const float *__restrict__ gamma,    // [K]
     float eps, const uint4 *__restrict__ w4,  // [nquads][KB]
-    float w_scale, int K, int KB, int N, int nquads, const float *residual, float *out) {
+    float w_scale, int K, int KB, int N, int nquads,
+    int vec /* N % 4 == 0, residual and out 16-byte aligned */, const float *residual, float *out) {
     constexpr int kWaves = W, kThreads = W * 64;
     constexpr int QPB = kWaves / KS;
     extern __shared__ uint4 s_a[];  // KB staged activation blocks (4-bit planes)
@@ -135,6 +136,17 @@ __global__ __launch_bounds__(W * 64) void bitlinear_gemv_kernel(
     for (int it = 0; it < L; ++it) {
         const int kb = sl_lo + it * 64 + lane;
         w[it] = wq[kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)];
+    }
+    // The residual the epilogue adds, requested behind the weights (one broadcast read per
+    // wave) instead of at the very end, where its round trip would be exposed.
+    float4 res4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    float res1 = 0.0f;
+    if (residual) {
+        if (KS == 1) {
+            if (vec) res4 = *reinterpret_cast<const float4 *>(residual + (size_t)min(quad * 4, N - 4));
+        } else if (tid < QPB * 4) {
+            res1 = residual[min((int)blockIdx.x * QPB * 4 + tid, N - 1)];
+        }
     }
     __builtin_amdgcn_sched_barrier(0);
 
@@ -235,19 +247,29 @@ __global__ __launch_bounds__(W * 64) void bitlinear_gemv_kernel(
 #pragma unroll
     for (int c = 0; c < 4; ++c) tot[c] = wave_total_lane63(hi[c] * 16 + lo[c]);
 
-    auto finish = [&](int n, int total) {
+    auto value = [&](int total) {
         total -= rowsum;
-        float r = (float)total * act_scale;  // kernels.rs:168, left to right
-        r = r * w_scale;
-        if (residual) r = residual[n] + r;
-        out[n] = r;
+        const float r = (float)total * act_scale;  // kernels.rs:168, left to right
+        return r * w_scale;
     };
     if (KS == 1) {
         if (lane == 63 && active) {
+            if (vec) {
+                // one 16-byte store: the stores end the launch, every instruction's round trip counts
+                if (quad * 4 < N) {  // quads of the column padding write nothing
+                    float4 r = make_float4(value(tot[0]), value(tot[1]), value(tot[2]), value(tot[3]));
+                    if (residual) r = make_float4(res4.x + r.x, res4.y + r.y, res4.z + r.z, res4.w + r.w);
+                    *reinterpret_cast<float4 *>(out + (size_t)quad * 4) = r;
+                }
+            } else {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int n = quad * 4 + c;
-                if (n < N) finish(n, tot[c]);
+                for (int c = 0; c < 4; ++c) {
+                    const int n = quad * 4 + c;
+                    if (n < N) {
+                        const float r = value(tot[c]);
+                        out[n] = residual ? residual[n] + r : r;
+                    }
+                }
             }
         }
     } else {
@@ -263,7 +285,8 @@ __global__ __launch_bounds__(W * 64) void bitlinear_gemv_kernel(
                 int total = 0;
 #pragma unroll
                 for (int s = 0; s < KS; ++s) total += s_part[(ql * KS + s) * 4 + c];
-                finish(n, total);
+                const float r = value(total);
+                out[n] = residual ? res1 + r : r;
             }
         }
     }
@@ -274,7 +297,7 @@ struct Args {
     float eps;
     const uint4 *w4;
     float w_scale;
-    int K, KB, N, nquads;
+    int K, KB, N, nquads, vec;
     const float *residual;
     float *out;
 };
@@ -285,10 +308,10 @@ void launch_w(hipStream_t stream, const Args &a) {
     dim3 grid((unsigned)((a.nquads + QPB - 1) / QPB));
     if (a.K <= 1024 * W)
         bitlinear_gemv_kernel<KS, L, SWIGLU, W, 1><<<grid, dim3(W * 64), (size_t)a.KB * 16, stream>>>(
-            a.x, a.gamma, a.eps, a.w4, a.w_scale, a.K, a.KB, a.N, a.nquads, a.residual, a.out);
+            a.x, a.gamma, a.eps, a.w4, a.w_scale, a.K, a.KB, a.N, a.nquads, a.vec, a.residual, a.out);
     else
         bitlinear_gemv_kernel<KS, L, SWIGLU, W, 2><<<grid, dim3(W * 64), (size_t)a.KB * 16, stream>>>(
-            a.x, a.gamma, a.eps, a.w4, a.w_scale, a.K, a.KB, a.N, a.nquads, a.residual, a.out);
+            a.x, a.gamma, a.eps, a.w4, a.w_scale, a.K, a.KB, a.N, a.nquads, a.vec, a.residual, a.out);
 }
 
 template <int KS, int L, bool SWIGLU>
@@ -357,6 +380,7 @@ extern "C" int rbn_bitlinear_gemv_f32(rbn_ctx *ctx, const float *d_x, const floa
     a.nquads = (int)(rbn_npad(N) / 4);
     a.residual = d_residual;
     a.out = d_out;
+    a.vec = N % 4 == 0 && (((uintptr_t)d_residual | (uintptr_t)d_out) & 15u) == 0;
     if (d_gate_up)
         launch_ks<true>(ctx->stream, a);
     else

@@ -63,13 +63,16 @@ __device__ __forceinline__ uint4 to_nibble_planes(uint4 a) {
 }
 
 // MT tokens, KS waves per column quad, L weight loads in flight per lane and round.
-template <int MT, int KS, int L>
+// EXACT: the k-blocks fit one pass and are a multiple of 64 * L, so no index of the
+// loop needs a clamp and no block a mask.
+template <int MT, int KS, int L, bool EXACT>
 __global__ __launch_bounds__(kThreads) void gemv_t2_i8_kernel(
     const uint4 *__restrict__ q4,         // [M][KB]: 16 int8 each
     const float *__restrict__ act_scale,  // [M]
     const int32_t *__restrict__ rowsum,   // [M]
     const uint4 *__restrict__ w4,         // [nquads][KB]
     float w_scale, int M, int KB, int KC /* k-blocks staged per pass */, int N, int nquads,
+    int vec_store /* N % 4 == 0 and the outputs are 16-byte aligned */,
     int32_t *__restrict__ acc_out, float *__restrict__ out) {
     constexpr int QPB = kWaves / KS;  // quads per workgroup
     extern __shared__ uint4 s_a[];  // MT * KC staged activation blocks (4-bit planes)
@@ -82,6 +85,15 @@ __global__ __launch_bounds__(kThreads) void gemv_t2_i8_kernel(
     const bool active = quad < nquads;
     quad = active ? quad : nquads - 1;
     const uint4 *wq = w4 + (size_t)quad * KB;
+
+    // epilogue scalars, fetched while the weights are in flight (spare token rows repeat the last)
+    int rs_m[MT];
+    float as_m[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        rs_m[m] = rowsum[min(m, M - 1)];
+        as_m[m] = act_scale[min(m, M - 1)];
+    }
 
     int hi[MT][4], lo[MT][4];
 #pragma unroll
@@ -118,7 +130,7 @@ __global__ __launch_bounds__(kThreads) void gemv_t2_i8_kernel(
         for (int it = 0; it < L; ++it) {
             const int kb = sl_lo + it * 64 + lane;
             // a lane past its slice re-reads its first block (a cache hit) and adds 0
-            w[it] = wq[kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)];
+            w[it] = wq[EXACT || kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)];
         }
         __builtin_amdgcn_sched_barrier(0);
         if (kc != 0) __syncthreads();  // everyone is done reading the previous pass
@@ -139,8 +151,8 @@ __global__ __launch_bounds__(kThreads) void gemv_t2_i8_kernel(
 #pragma unroll
             for (int it = 0; it < L; ++it) {
                 const int kb = r0 + it * 64 + lane;
-                const uint32_t keep = kb < sl_hi ? 0x33333333u : 0u;
-                const int a_idx = min(kb, sl_hi - 1) - kc;
+                const uint32_t keep = EXACT || kb < sl_hi ? 0x33333333u : 0u;
+                const int a_idx = EXACT ? kb : min(kb, sl_hi - 1) - kc;
                 const uint32_t ww[4] = {wr[it].x, wr[it].y, wr[it].z, wr[it].w};
                 uint32_t ev[4], od[4];
 #pragma unroll
@@ -169,7 +181,7 @@ __global__ __launch_bounds__(kThreads) void gemv_t2_i8_kernel(
 #pragma unroll
             for (int it = 0; it < L; ++it) {
                 const int kb = r0 + 64 * L + it * 64 + lane;
-                wn[it] = wq[kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)];
+                wn[it] = wq[EXACT || kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)];
             }
             consume(w, r0);
 #pragma unroll
@@ -191,17 +203,35 @@ __global__ __launch_bounds__(kThreads) void gemv_t2_i8_kernel(
 #pragma unroll
             for (int m = 0; m < MT; ++m) {
                 if (m >= M) break;
-                const int rs = rowsum[m];
-                const float as = act_scale[m];
+                const int rs = rs_m[m];
+                const float as = as_m[m];
+                if (vec_store) {
+                    // one 16-byte store per token instead of four: the stores sit at the very end
+                    // of the launch, where each instruction's round trip is exposed
+                    int t4[4];
+                    float r4[4];
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const int n = quad * 4 + c;
-                    if (n < N) {
-                        const int total = tot[m][c] - rs;
-                        if (acc_out) acc_out[(size_t)m * N + n] = total;
-                        float r = (float)total * as;  // kernels.rs:168, left to right
-                        r = r * w_scale;
-                        out[(size_t)m * N + n] = r;
+                    for (int c = 0; c < 4; ++c) {
+                        t4[c] = tot[m][c] - rs;
+                        const float r = (float)t4[c] * as;  // kernels.rs:168, left to right
+                        r4[c] = r * w_scale;
+                    }
+                    const size_t at = (size_t)m * N + (size_t)quad * 4;
+                    if (quad * 4 < N) {  // quads of the column padding write nothing
+                        if (acc_out) *(int4 *)(acc_out + at) = make_int4(t4[0], t4[1], t4[2], t4[3]);
+                        *(float4 *)(out + at) = make_float4(r4[0], r4[1], r4[2], r4[3]);
+                    }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const int n = quad * 4 + c;
+                        if (n < N) {
+                            const int total = tot[m][c] - rs;
+                            if (acc_out) acc_out[(size_t)m * N + n] = total;
+                            float r = (float)total * as;  // kernels.rs:168, left to right
+                            r = r * w_scale;
+                            out[(size_t)m * N + n] = r;
+                        }
                     }
                 }
             }
@@ -238,7 +268,7 @@ struct Args {
     const int32_t *rowsum;
     const uint4 *w4;
     float w_scale;
-    int M, KB, KC, N, nquads;
+    int M, KB, KC, N, nquads, vec_store, exact;
     int32_t *acc;
     float *out;
 };
@@ -248,8 +278,16 @@ void launch(hipStream_t stream, const Args &a) {
     constexpr int QPB = kWaves / KS;
     dim3 grid((unsigned)((a.nquads + QPB - 1) / QPB));
     const size_t lds = (size_t)MT * a.KC * 16;
-    gemv_t2_i8_kernel<MT, KS, L><<<grid, dim3(kThreads), lds, stream>>>(
-        a.q4, a.act_scale, a.rowsum, a.w4, a.w_scale, a.M, a.KB, a.KC, a.N, a.nquads, a.acc, a.out);
+    if constexpr (KS == 1 && MT <= 4) {
+        if (a.exact && a.KC == a.KB && a.KB % (64 * L) == 0) {
+            gemv_t2_i8_kernel<MT, KS, L, true><<<grid, dim3(kThreads), lds, stream>>>(
+                a.q4, a.act_scale, a.rowsum, a.w4, a.w_scale, a.M, a.KB, a.KC, a.N, a.nquads, a.vec_store, a.acc,
+                a.out);
+            return;
+        }
+    }
+    gemv_t2_i8_kernel<MT, KS, L, false><<<grid, dim3(kThreads), lds, stream>>>(
+        a.q4, a.act_scale, a.rowsum, a.w4, a.w_scale, a.M, a.KB, a.KC, a.N, a.nquads, a.vec_store, a.acc, a.out);
 }
 
 template <int MT, int KS>
@@ -299,14 +337,24 @@ extern "C" int rbn_gemv_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_ac
     a.nquads = (int)(rbn_npad(N) / 4);
     a.acc = d_acc;
     a.out = d_out;
+    a.vec_store = N % 4 == 0 && (((uintptr_t)d_out | (uintptr_t)d_acc) & 15u) == 0;
+    a.exact = 1;
     const int mt = M == 1 ? 1 : M == 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
     // k-blocks whose staged activations fit the LDS budget in one pass
     const int kc_cap = kLdsBudget / 16 / mt;
     a.KC = a.KB < kc_cap ? a.KB : kc_cap;
     // Waves per quad: enough wavefronts to cover the chip (256 CUs x 4 SIMDs, a few waves
-    // each) without shrinking a wave's share of k below one round.
+    // each) without shrinking a wave's share of k below one round.  One token tolerates
+    // shorter shares than several (measured crossovers).
     int ks = 1;
-    while (ks < 4 && (long long)a.nquads * ks < 2048 && a.KB / (ks * 2) >= 128) ks *= 2;
+    if (M == 1) {
+        if (a.nquads <= 1024 && a.KB >= 640)
+            ks = 4;
+        else if ((a.nquads <= 1024 && a.KB >= 160) || (a.nquads <= 2048 && a.KB >= 512))
+            ks = 2;
+    } else {
+        while (ks < 4 && (long long)a.nquads * ks < 2048 && a.KB / (ks * 2) >= 128) ks *= 2;
+    }
     switch (mt) {
         case 1: launch_ks<1>(ctx->stream, a, ks); break;
         case 2: launch_ks<2>(ctx->stream, a, ks); break;

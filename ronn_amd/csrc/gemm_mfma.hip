@@ -438,11 +438,14 @@ extern "C" int rbn_gemm_t2_i8_mfma(rbn_ctx *ctx, const int8_t *d_q, const float 
 }
 
 extern "C" int rbn_matmul_kernel_choice(uint64_t M, uint64_t K, uint64_t N) {
-    // measured crossovers: the dot-instruction GEMV wins up to three tokens; the streaming
-    // small-batch kernel up to 32 tokens (16 on very large matrices) and, on small matrices,
-    // up to its limit of 64; the tiled kernel beyond
-    if (M <= 3) return RBN_KERNEL_GEMV;
+    // measured crossovers: the dot-instruction GEMV wins for one and two tokens (its time
+    // grows with M, so not for two tokens on a wide matrix with a short k) and up to four
+    // tokens on small matrices; the streaming small-batch kernel up to 32 tokens (16 on very
+    // large matrices) and, on small matrices, up to its limit of 64; the tiled kernel beyond
     const uint64_t kn = K * N;
+    if (M == 1) return RBN_KERNEL_GEMV;
+    if (M == 2 && !(K <= 3072 && kn >= (1ull << 25))) return RBN_KERNEL_GEMV;
+    if (M >= 3 && M <= 4 && kn <= (1ull << 24)) return RBN_KERNEL_GEMV;
     if (M <= 16 || (M <= 32 && kn < (1ull << 27)) || (M <= RBN_SKINNY_MAX_M && kn < (1ull << 25)))
         return RBN_KERNEL_SKINNY;
     return RBN_KERNEL_MFMA;

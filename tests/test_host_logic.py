@@ -37,13 +37,16 @@ def test_library_exports_every_declared_symbol(lib):
 
 
 def test_matmul_dispatch_rule(lib):
-    # gemv up to 3 tokens; the small-batch kernel up to 16, 32 or 64 by the size of the matrix
+    # gemv for one or two tokens and for up to four on small matrices; the small-batch kernel
+    # up to 16, 32 or 64 by the size of the matrix
     choice = lib.rbn_matmul_kernel_choice
     GEMV, SKINNY, MFMA = 0, 1, 2
-    assert [choice(m, 4096, 11008) for m in (1, 3, 4, 16, 32, 33, 64, 65)] == \
-        [GEMV, GEMV, SKINNY, SKINNY, SKINNY, MFMA, MFMA, MFMA]
-    assert [choice(m, 8192, 28672) for m in (1, 8, 16, 17, 64)] == [GEMV, SKINNY, SKINNY, MFMA, MFMA]
-    assert [choice(m, 4096, 4096) for m in (4, 64, 65, 2048)] == [SKINNY, SKINNY, MFMA, MFMA]
+    assert [choice(m, 4096, 11008) for m in (1, 2, 3, 4, 16, 32, 33, 64, 65)] == \
+        [GEMV, GEMV, SKINNY, SKINNY, SKINNY, SKINNY, MFMA, MFMA, MFMA]
+    assert [choice(m, 8192, 28672) for m in (1, 2, 3, 8, 16, 17, 64)] == \
+        [GEMV, GEMV, SKINNY, SKINNY, SKINNY, MFMA, MFMA]
+    assert [choice(m, 4096, 4096) for m in (3, 4, 5, 64, 65, 2048)] == [GEMV, GEMV, SKINNY, SKINNY, MFMA, MFMA]
+    assert [choice(m, 2560, 13824) for m in (1, 2)] == [GEMV, SKINNY]   # short k, wide: two tokens stream
 
 
 def test_provider_abi_exports(lib):

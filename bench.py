@@ -30,7 +30,7 @@ INT8_PEAK_TOPS = 5000.0     # MI355X published dense int8 MFMA rate (5.0 POP/s)
 MALL_BYTES = 256 << 20
 # HBM bytes per launch of the headline GEMV, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a
 # 256 MiB copy (profiles/gemv_m1_k4096_n11008.md)
-GEMV_HEADLINE_TRAFFIC_BYTES = 11424227
+GEMV_HEADLINE_TRAFFIC_BYTES = 11406785
 
 
 def gemv_bytes(M, K, N):
@@ -319,7 +319,7 @@ def main():
                    "compute_units": info["compute_units"], "clock_mhz": info["clock_khz"] / 1000.0},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": GEMV_HEADLINE_TRAFFIC_BYTES,
-                     "kernel": "gemv_t2_i8_kernel<1, 1, 4>", "bytes_per_launch": bytes_per_launch,
+                     "kernel": "gemv_t2_i8_kernel<1, 1, 4, true>", "bytes_per_launch": bytes_per_launch,
                      "us_per_launch": ev_ms * 1e3},
     }
 

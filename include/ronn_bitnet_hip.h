@@ -189,7 +189,8 @@ int rbn_act_quant_ternary(rbn_ctx *ctx, const float *d_x, uint64_t M, uint64_t K
  * once with int8 dot instructions.  rbn_gemm_t2_i8_skinny: small batches
  * (M <= RBN_SKINNY_MAX_M), the same streaming read with 16x16x64 int8 MFMA doing
  * the dot products.  rbn_gemm_t2_i8_mfma: prefill regime, 128x256 tiles of int8
- * MFMA.  rbn_matmul_t2_i8 picks one by M and K*N (1..3: gemv; skinny up to 16 tokens, up to 32
+ * MFMA.  rbn_matmul_t2_i8 picks one by M, K and N (gemv for 1 and 2 tokens - not for 2 when
+ * K <= 3072 and K*N >= 2^25 - and up to 4 when K*N <= 2^24; skinny up to 16 tokens, up to 32
  * when K*N < 2^27, up to 64 when K*N < 2^25; mfma otherwise).
  * All three give identical results. */
 #define RBN_GEMV_MAX_M 16

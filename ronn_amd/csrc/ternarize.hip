@@ -6,6 +6,7 @@
 // TernaryTensor::get_value (:275-291) in crates/ronn-providers/src/bitnet/.
 #include <cmath>
 #include <cstring>
+#include <type_traits>
 
 #include "common.hpp"
 #include "seqsum_core.h"
@@ -425,35 +426,70 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         const uint32_t chunk = (nblocks + 1023u) / 1024u;
         const uint32_t lo = t * chunk;
         const uint32_t hi = lo + chunk < nblocks ? lo + chunk : nblocks;
-        // batches of eight loads in flight (a dependent loop would pay one round trip per map)
+        // A thread's maps are loaded once, all loads in flight, and kept in registers for
+        // both walks (composition, then the search for the crossing) when there are at
+        // most 32 of them (windows up to 32768 blocks); longer chunks are walked twice in
+        // batches of eight.  Spare slots re-read the chunk's last map and are skipped.
         SeqMap mine = seq_identity();
-        for (uint32_t b0 = lo; b0 < hi; b0 += 8) {
-            SeqMap mm[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) mm[i] = maps[b0 + i < hi ? b0 + i : hi - 1];
-#pragma unroll
-            for (int i = 0; i < 8; ++i)
-                if (b0 + i < hi) mine = seq_compose(mine, mm[i]);
-        }
+        uint32_t k = 0, cand = 0xffffffffu, cand_k = 0;
         if (t == 0) s_first = 0xffffffffu;
-        SeqMap all;
-        const SeqMap before = seq_block_before<16>(mine, s_w, &all);
-        uint32_t k = seq_apply(before, k0);
-        uint32_t cand = 0xffffffffu, cand_k = 0;
-        if (k < SEQ_K_LIMIT) {
-            for (uint32_t b0 = lo; b0 < hi && cand == 0xffffffffu; b0 += 8) {
+        auto walk_cached = [&](auto size_tag) {
+            constexpr int C = decltype(size_tag)::value;
+            SeqMap mm[C];
+#pragma unroll
+            for (int i = 0; i < C; ++i) mm[i] = maps[lo + i < hi ? lo + i : (hi > 0 ? hi - 1 : 0)];
+#pragma unroll
+            for (int i = 0; i < C; ++i)
+                if (lo + i < hi) mine = seq_compose(mine, mm[i]);
+            SeqMap all;
+            const SeqMap before = seq_block_before<16>(mine, s_w, &all);
+            k = seq_apply(before, k0);
+            if (k < SEQ_K_LIMIT) {
+#pragma unroll
+                for (int i = 0; i < C; ++i) {
+                    if (lo + i < hi && cand == 0xffffffffu) {
+                        const uint32_t k2 = seq_apply(mm[i], k);
+                        if (k2 >= SEQ_K_LIMIT) {
+                            cand = lo + i;
+                            cand_k = k;
+                        } else {
+                            k = k2;
+                        }
+                    }
+                }
+            }
+        };
+        if (chunk <= 8u) {
+            walk_cached(std::integral_constant<int, 8>{});
+        } else if (chunk <= 32u) {
+            walk_cached(std::integral_constant<int, 32>{});
+        } else {
+            for (uint32_t b0 = lo; b0 < hi; b0 += 8) {
                 SeqMap mm[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) mm[i] = maps[b0 + i < hi ? b0 + i : hi - 1];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    if (b0 + i < hi && cand == 0xffffffffu) {
-                        const uint32_t k2 = seq_apply(mm[i], k);
-                        if (k2 >= SEQ_K_LIMIT) {
-                            cand = b0 + i;
-                            cand_k = k;
-                        } else {
-                            k = k2;
+                for (int i = 0; i < 8; ++i)
+                    if (b0 + i < hi) mine = seq_compose(mine, mm[i]);
+            }
+            SeqMap all;
+            const SeqMap before = seq_block_before<16>(mine, s_w, &all);
+            k = seq_apply(before, k0);
+            if (k < SEQ_K_LIMIT) {
+                for (uint32_t b0 = lo; b0 < hi && cand == 0xffffffffu; b0 += 8) {
+                    SeqMap mm[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) mm[i] = maps[b0 + i < hi ? b0 + i : hi - 1];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        if (b0 + i < hi && cand == 0xffffffffu) {
+                            const uint32_t k2 = seq_apply(mm[i], k);
+                            if (k2 >= SEQ_K_LIMIT) {
+                                cand = b0 + i;
+                                cand_k = k;
+                            } else {
+                                k = k2;
+                            }
                         }
                     }
                 }
@@ -692,7 +728,12 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     // sizes the next one by the binades S still has to climb (a window ends where S leaves
     // its binade).
     const unsigned grid = (unsigned)(total_blocks < (uint64_t)kMapGrid ? total_blocks : (uint64_t)kMapGrid);
-    int batch = 4;
+    // first batch: S of similar terms climbs one binade per doubling of the position, plus the
+    // first block's window and two spare (a spare pair of launches returns at once: 4 us;
+    // another look by the host costs 10-25 us)
+    int batch = 3;
+    for (uint64_t b = total_blocks; b > 1; b >>= 1) ++batch;
+    batch = batch > 24 ? 24 : batch;
     for (;;) {
         for (int i = 0; i < batch; ++i) {
             seq_block_maps_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(

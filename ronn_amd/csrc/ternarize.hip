@@ -348,20 +348,28 @@ __global__ __launch_bounds__(kBlock) void sum_u64_kernel(const unsigned long lon
 // composition of everything BEFORE this thread, and in *total the composition of all; NW = waves
 // that carry values (the others pass the identity).  One __syncthreads inside: every thread of
 // the workgroup must call it, and s_w must not be touched again before the next barrier.
+// A SeqMap from another lane by a DPP move: lanes without a source (and rows outside the
+// mask) read zeros, which is the identity map.
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ SeqMap seq_dpp(SeqMap m) {
+    SeqMap o;
+    o.d0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m.d0, CTRL, ROWMASK, 0xf, true);
+    o.d1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m.d1, CTRL, ROWMASK, 0xf, true);
+    return o;
+}
+
 template <int NW>
 __device__ __forceinline__ SeqMap seq_block_before(SeqMap m, SeqMap *s_w, SeqMap *total) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int off = 1; off < 64; off <<= 1) {
-        SeqMap o;
-        o.d0 = __shfl_up(m.d0, off);
-        o.d1 = __shfl_up(m.d1, off);
-        if (lane >= off) m = seq_compose(o, m);
-    }
+    // inclusive scan of the wave: inside rows of 16 lanes, then across the rows
+    m = seq_compose(seq_dpp<0x111, 0xf>(m), m);  // row_shr:1
+    m = seq_compose(seq_dpp<0x112, 0xf>(m), m);  // row_shr:2
+    m = seq_compose(seq_dpp<0x114, 0xf>(m), m);  // row_shr:4
+    m = seq_compose(seq_dpp<0x118, 0xf>(m), m);  // row_shr:8
+    m = seq_compose(seq_dpp<0x142, 0xa>(m), m);  // row_bcast15: rows 1, 3 absorb the row before
+    m = seq_compose(seq_dpp<0x143, 0xc>(m), m);  // row_bcast31: rows 2, 3 absorb rows 0-1
     if (lane == 63 && wave < NW) s_w[wave] = m;
-    SeqMap ex;  // exclusive inside the wave
-    ex.d0 = __shfl_up(m.d0, 1);
-    ex.d1 = __shfl_up(m.d1, 1);
-    if (lane == 0) ex = seq_identity();
+    const SeqMap ex = seq_dpp<0x138, 0xf>(m);  // wave_shr:1: exclusive inside the wave, lane 0 reads the identity
     __syncthreads();
     SeqMap pre = seq_identity(), tot = seq_identity();
 #pragma unroll
@@ -387,13 +395,17 @@ __device__ __forceinline__ SeqMap seq_block_before(SeqMap m, SeqMap *s_w, SeqMap
 // host mailbox (the host reads it after synchronising: it sizes the next window).
 __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     const SeqMap *__restrict__ maps, const float *__restrict__ x, uint64_t n, uint64_t total_blocks,
-    int use_mask, float thr, SeqState *__restrict__ state, SeqState *__restrict__ host_copy) {
+    int use_mask, float thr, SeqState *__restrict__ state, SeqState *__restrict__ host_copy,
+    int mirror /* the last launch of a batch: the host reads the state after it */) {
     __shared__ SeqMap s_w[16];
     __shared__ unsigned s_first;
     __shared__ uint32_t s_cross_block, s_cross_k;
     __shared__ uint32_t s_bits_now;
     const uint32_t t = threadIdx.x;
-    if (state->done) return;
+    if (state->done) {
+        if (mirror && t == 0) *host_copy = *state;
+        return;
+    }
     const uint32_t nblocks = state->win;
     const uint64_t pos0 = state->pos;
     const uint64_t first = pos0 * kSeqTile;
@@ -418,7 +430,7 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         const uint64_t seen = pos0 + nblocks, before = state->fresh_from;
         next.fresh_from = seen > before ? seen : before;
         *state = next;
-        *host_copy = next;
+        if (mirror) *host_copy = next;  // a store to pinned host memory: only when somebody will look
     };
 
     // ---- (1) scan -----------------------------------------------------------------------
@@ -739,7 +751,7 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
             seq_block_maps_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
                 d_x, n, use_mask, thr, &scr->seq, maps, (uint32_t *)d_packed, count_parts);
             seq_scan_replay_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(
-                maps, d_x, n, total_blocks, use_mask, thr, &scr->seq, h_state);
+                maps, d_x, n, total_blocks, use_mask, thr, &scr->seq, h_state, i == batch - 1);
         }
         RBN_HIP(hipGetLastError());
         RBN_HIP(hipStreamSynchronize(ctx->stream));

@@ -227,6 +227,16 @@ struct SeqState {
     uint64_t fresh_from;  // blocks from here on have not been seen by any window yet
 };
 
+// A SeqMap from another lane by a DPP move: lanes without a source (and rows outside the
+// mask) read zeros, which is the identity map.
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ SeqMap seq_dpp(SeqMap m) {
+    SeqMap o;
+    o.d0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m.d0, CTRL, ROWMASK, 0xf, true);
+    o.d1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m.d1, CTRL, ROWMASK, 0xf, true);
+    return o;
+}
+
 // One SeqMap per block of 4096 elements, valid for a state of biased exponent `es`.
 // The window and the exponent come from the state; the grid strides over the window's blocks.
 // With `packed` given (masked sums only: thr is the ternary threshold) the kernel also packs
@@ -287,14 +297,15 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
         }
         if (fresh && base < n) packed[base >> 4] = word;  // tail bits stay zero
     }
-    // ordered tree over the wave: lane l absorbs lane l+off (its right neighbour)
-    for (int off = 1; off < 64; off <<= 1) {
-        SeqMap o;
-        o.d0 = __shfl_down(m.d0, off);
-        o.d1 = __shfl_down(m.d1, off);
-        m = seq_compose(m, o);
-    }
-    if ((threadIdx.x & 63) == 0) s_wave[threadIdx.x >> 6] = m;
+    // ordered reduction of the wave by DPP moves (each lane absorbs what lies to its left):
+    // lane 63 ends up with the map of all 1024 elements
+    m = seq_compose(seq_dpp<0x111, 0xf>(m), m);  // row_shr:1
+    m = seq_compose(seq_dpp<0x112, 0xf>(m), m);  // row_shr:2
+    m = seq_compose(seq_dpp<0x114, 0xf>(m), m);  // row_shr:4
+    m = seq_compose(seq_dpp<0x118, 0xf>(m), m);  // row_shr:8
+    m = seq_compose(seq_dpp<0x142, 0xa>(m), m);  // row_bcast15
+    m = seq_compose(seq_dpp<0x143, 0xc>(m), m);  // row_bcast31
+    if ((threadIdx.x & 63) == 63) s_wave[threadIdx.x >> 6] = m;
     __syncthreads();
     if (threadIdx.x == 0) {
         SeqMap t = s_wave[0];
@@ -348,16 +359,6 @@ __global__ __launch_bounds__(kBlock) void sum_u64_kernel(const unsigned long lon
 // composition of everything BEFORE this thread, and in *total the composition of all; NW = waves
 // that carry values (the others pass the identity).  One __syncthreads inside: every thread of
 // the workgroup must call it, and s_w must not be touched again before the next barrier.
-// A SeqMap from another lane by a DPP move: lanes without a source (and rows outside the
-// mask) read zeros, which is the identity map.
-template <int CTRL, int ROWMASK>
-__device__ __forceinline__ SeqMap seq_dpp(SeqMap m) {
-    SeqMap o;
-    o.d0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m.d0, CTRL, ROWMASK, 0xf, true);
-    o.d1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m.d1, CTRL, ROWMASK, 0xf, true);
-    return o;
-}
-
 template <int NW>
 __device__ __forceinline__ SeqMap seq_block_before(SeqMap m, SeqMap *s_w, SeqMap *total) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;

@@ -192,7 +192,10 @@ int rbn_act_quant_ternary(rbn_ctx *ctx, const float *d_x, uint64_t M, uint64_t K
  * MFMA.  rbn_matmul_t2_i8 picks one by M, K and N (gemv for 1 and 2 tokens - not for 2 when
  * K <= 3072 and K*N >= 2^25 - and up to 4 when K*N <= 2^24; skinny up to 16 tokens, up to 32
  * when K*N < 2^27, up to 64 when K*N < 2^25; mfma otherwise).
- * All three give identical results. */
+ * All three give identical results.
+ * d_q and d_tiled must be 16-byte aligned; so must d_out and d_acc for every entry point
+ * except rbn_gemv_t2_i8, which accepts any float/int32 alignment there (memory from
+ * rbn_malloc is 256-byte aligned).  A misaligned pointer is RBN_ERR_INVALID. */
 #define RBN_GEMV_MAX_M 16
 #define RBN_SKINNY_MAX_M 64
 int rbn_gemv_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,

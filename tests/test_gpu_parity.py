@@ -381,7 +381,7 @@ def test_skinny_saturated_activations(ctx):
     assert np.abs(res[1]).max() > 127 * 100
 
 
-@pytest.mark.parametrize("M", [1, 2, 16, 17, 64, 65, 128])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 5, 16, 17, 64, 65, 128])
 def test_matmul_dispatch_agrees_across_kernels(ctx, M):
     # rbn_matmul_t2_i8 picks gemv / skinny / mfma by M; every kernel that accepts the shape
     # must return the same bits
@@ -398,6 +398,19 @@ def test_matmul_dispatch_agrees_across_kernels(ctx, M):
     for fn in fns:
         got = run_matmul(ctx, fn, x, w)
         assert (got[1] == ref[1]).all() and same_bits(got[0], ref[0])
+
+
+def test_matmul_two_tokens_wide_short_k(ctx):
+    # two tokens go to the streaming kernel when k is short and the matrix wide, to the GEMV
+    # otherwise: same bits either way (2560 x 13824 is the decoder's gate/up projection)
+    M, K, N = 2, 2560, 13824
+    assert ctx.lib.rbn_matmul_kernel_choice(M, K, N) == 1 and ctx.lib.rbn_matmul_kernel_choice(M, 4096, N) == 0
+    x = synth_normal(0x5EED0031, 1.0, (M, K))
+    w = synth_normal(0x5EED1031, 0.02, (K, N))
+    ref = run_matmul(ctx, ctx.matmul, x, w)
+    check_against_oracle(x, w, *ref, literal=False)
+    got = run_matmul(ctx, ctx.gemv, x, w)
+    assert (got[1] == ref[1]).all() and same_bits(got[0], ref[0])
 
 
 def test_gemm_mfma_saturated_activations(ctx):

@@ -492,7 +492,7 @@ __global__ __launch_bounds__(256) void attention_mfma_kernel(
 //    for P.V, so a block is one round trip of 20 loads per lane.
 //  * The workgroups of a head publish (max, sum, out[128]) as device-scope stores, draw a
 //    ticket, and the last one combines and writes the result: no second launch, nobody waits.
-constexpr int kSplits = 8;
+constexpr int kSplits = 12;
 constexpr int kPartial = 132;  // floats per partial: out[128], max, sum, padding
 __global__ __launch_bounds__(256) void attention_decode_kernel(
     const float *__restrict__ qkv, const int32_t *__restrict__ pos, int heads, float theta,

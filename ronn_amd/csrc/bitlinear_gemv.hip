@@ -318,9 +318,10 @@ template <int KS, int L, bool SWIGLU>
 void launch(hipStream_t stream, const Args &a) {
     // Every workgroup repeats the normalisation of the whole row: eight waves halve that
     // work per thread and the number of workgroups re-reading the row.  It pays for long
-    // rows (K > 4096: one block per thread again) and for wide matrices (measured: 6912 x
-    // 2560 8.3 -> 5.6 us, 2560 x 13824 6.4 -> 6.1 us; 2560 x 2560 is faster with four).
-    if (a.K > 4096 || a.nquads >= 3072)
+    // rows (K > 4096: one block per thread again; 6912 x 2560 8.3 -> 5.6 us); at K = 2560
+    // four waves are faster whatever the width (a decode step with 2560 x 13824 and
+    // 2560 x 32000 on eight waves: 0.737 ms, on four: 0.731 ms).
+    if (a.K > 4096)
         launch_w<KS, L, SWIGLU, 8>(stream, a);
     else
         launch_w<KS, L, SWIGLU, 4>(stream, a);

@@ -177,7 +177,7 @@ def time_decoder(ctx, prompt_len=512, new_tokens=128, use_graph=True):
     return {"config": dataclass_dict(cfg), "prompt_tokens": prompt_len, "new_tokens": new_tokens,
             "decode_tok_per_s": new_tokens / dt, "ms_per_token": per_tok * 1e3,
             "prefill_ms": t_prefill * 1e3, "prefill_tok_per_s": prompt_len / t_prefill,
-            "weight_init_s": t_init, "launches_per_token": 5 * cfg.layers + 4,
+            "weight_init_s": t_init, "launches_per_token": 5 * cfg.layers + 2,
             "bytes_per_token": {"packed_weights": w_bytes, "kv_cache_f16_avg": kv_bytes},
             "GBps": (w_bytes + kv_bytes) / per_tok / 1e9,
             "frac_hbm_peak": (w_bytes + kv_bytes) / per_tok / 1e9 / HBM_PEAK_GBS,

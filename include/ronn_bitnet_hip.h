@@ -273,6 +273,13 @@ int rbn_swiglu_f32(rbn_ctx *ctx, const float *d_gate_up, uint64_t M, uint64_t F,
  * is given the index is also written to d_history[*d_history_pos]. */
 int rbn_argmax_f32(rbn_ctx *ctx, const float *d_values, uint64_t n, int32_t *d_index,
                    int32_t *d_history, const int32_t *d_history_pos);
+/* The tail of a greedy decode step in one launch: *d_pos += 1; t = arg-max of the vocab
+ * logits (lowest index among equals); *d_token = t; d_history[*d_pos] = t; d_x[0..H) =
+ * d_table[t, :] (the next step's embedding).  No counterpart in the reference (decoder
+ * harness). */
+int rbn_greedy_next_f32(rbn_ctx *ctx, const float *d_logits, uint64_t vocab, int32_t *d_token,
+                        int32_t *d_history, int32_t *d_pos, const float *d_table, uint64_t H,
+                        float *d_x);
 /* *d_value += delta (the position counter of a captured decode step). */
 int rbn_add_i32(rbn_ctx *ctx, int32_t *d_value, int32_t delta);
 /* Normal(0, sigma) values generated on the device (counter-based, f32 Box-Muller);

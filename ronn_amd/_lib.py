@@ -98,6 +98,7 @@ SIGNATURES = {
     "rbn_attention_decode_f16kv": (C.c_int, [_vp, _vp, _vp, _u64, _u64, C.c_float, _vp, _vp, _u64, _vp]),
     "rbn_swiglu_f32": (C.c_int, [_vp, _vp, _u64, _u64, _vp]),
     "rbn_argmax_f32": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _vp]),
+    "rbn_greedy_next_f32": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _vp, _vp, _u64, _vp]),
     "rbn_add_i32": (C.c_int, [_vp, _vp, C.c_int32]),
     "rbn_synth_normal_device_f32": (C.c_int, [_vp, _u64, C.c_float, _vp, _u64]),
     "rbn_probe_mfma_i8": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_double)]),

@@ -662,12 +662,18 @@ __global__ __launch_bounds__(kBlock) void swiglu_kernel(const float *__restrict_
 }
 
 // Index of the largest of n values (the lowest index among equals); one workgroup.
+// With `advance` the position counter hist_pos[0] is incremented first (the history slot is
+// the new position); with `table` the row of the chosen index is copied to x_out (the next
+// step's embedding): the tail of a greedy decode step in one launch.
 __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ v, int n,
                                                       int32_t *__restrict__ out,
                                                       int32_t *__restrict__ hist,
-                                                      const int32_t *__restrict__ hist_pos) {
+                                                      int32_t *__restrict__ hist_pos, int advance,
+                                                      const float *__restrict__ table, int H,
+                                                      float *__restrict__ x_out) {
     __shared__ float s_v[16];
     __shared__ int s_i[16];
+    __shared__ int s_pick;
     float best = -INFINITY;
     int bi = 0x7fffffff;
     auto take = [&](float x, int i) {
@@ -718,8 +724,17 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
             }
         bi = bi == 0x7fffffff ? 0 : bi;
         out[0] = bi;
-        if (hist) hist[hist_pos[0]] = bi;
+        if (hist) {
+            int p = hist_pos[0];
+            if (advance) hist_pos[0] = ++p;
+            hist[p] = bi;
+        }
+        s_pick = bi;
     }
+    if (table == nullptr) return;
+    __syncthreads();
+    const float *row = table + (size_t)s_pick * H;
+    for (int i = threadIdx.x; i < H; i += 1024) x_out[i] = row[i];
 }
 
 __global__ void add_i32_kernel(int32_t *p, int delta) { p[0] += delta; }
@@ -857,7 +872,21 @@ int rbn_argmax_f32(rbn_ctx *ctx, const float *d_values, uint64_t n, int32_t *d_i
     RBN_REQUIRE((d_history == nullptr) == (d_history_pos == nullptr),
                 "d_history and d_history_pos go together");
     argmax_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(d_values, (int)n, d_index, d_history,
-                                                          d_history_pos);
+                                                          const_cast<int32_t *>(d_history_pos), 0, nullptr,
+                                                          0, nullptr);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+int rbn_greedy_next_f32(rbn_ctx *ctx, const float *d_logits, uint64_t vocab, int32_t *d_token,
+                        int32_t *d_history, int32_t *d_pos, const float *d_table, uint64_t H,
+                        float *d_x) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(d_logits && d_token && d_history && d_pos && d_table && d_x && vocab > 0 && H > 0 &&
+                    vocab < (1ull << 31) && H < (1ull << 31),
+                "bad arguments in rbn_greedy_next_f32");
+    argmax_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(d_logits, (int)vocab, d_token, d_history, d_pos,
+                                                          1, d_table, (int)H, d_x);
     RBN_HIP(hipGetLastError());
     return RBN_OK;
 }

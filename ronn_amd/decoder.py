@@ -6,7 +6,7 @@ reference has no decoder (its BitNet provider stops at the matmul,
 crates/ronn-providers/src/bitnet/kernels.rs:134-178), so the layer formulas are the usual
 LLaMA / BitNet-b1.58 ones; tests/decoder_model.py restates them in numpy.
 
-A decode step is 124 kernel launches; it reads the position and the previous token from
+A decode step is 122 kernel launches; it reads the position and the previous token from
 device memory, so it is captured once in a HIP graph and replayed per token.
 """
 from __future__ import annotations
@@ -176,7 +176,6 @@ class BitNetDecoder:
         """forward(1) with five launches per layer: every BitLinear is one kernel, the
         residual additions ride on the o and down projections."""
         cfg, lib, hnd = self.cfg, self.lib, self.ctx.handle
-        check(lib.rbn_embed_f32(hnd, self.embed.ptr, self.tokens.ptr, 1, cfg.hidden, cfg.vocab, self.x.ptr))
         for i, b in enumerate(self.blocks):
             self._bitlinear1(b["wqkv"], b["g_attn"], self.qkv, x=self.x)
             check(lib.rbn_attention_decode_f16kv(hnd, self.qkv.ptr, self.pos.ptr, cfg.heads, cfg.head_dim,
@@ -186,9 +185,9 @@ class BitNetDecoder:
             self._bitlinear1(b["wgu"], b["g_ffn"], self.gu, x=self.x)
             self._bitlinear1(b["wdown"], b["g_ffn_sub"], self.x, gate_up=self.gu, residual=self.x)
         self._bitlinear1(self.lm_head, self.g_final, self.logits, x=self.x)
-        check(lib.rbn_add_i32(hnd, self.pos.ptr, 1))
-        check(lib.rbn_argmax_f32(hnd, self.logits.ptr, cfg.vocab, self.tokens.ptr, self.history.ptr,
-                                 self.pos.ptr))
+        # position + 1, arg-max, history, and the next step's embedding in one launch
+        check(lib.rbn_greedy_next_f32(hnd, self.logits.ptr, cfg.vocab, self.tokens.ptr, self.history.ptr,
+                                      self.pos.ptr, self.embed.ptr, cfg.hidden, self.x.ptr))
 
     def forward(self, M: int):
         """Tokens self.tokens[0:M] at positions *pos .. *pos+M-1; leaves the logits of the
@@ -250,6 +249,10 @@ class BitNetDecoder:
     def decode(self, n_tokens: int, use_graph: bool = True):
         """Greedy decoding of n_tokens more tokens; returns (tokens, seconds)."""
         g = self.capture_decode_step() if use_graph else None
+        # a step expects the embedding of the previous token in self.x (each step leaves the
+        # next one's there; after a prompt it has to be looked up once)
+        check(self.lib.rbn_embed_f32(self.ctx.handle, self.embed.ptr, self.tokens.ptr, 1, self.cfg.hidden,
+                                     self.cfg.vocab, self.x.ptr))
         self.ctx.sync()
         t0 = time.perf_counter()
         for _ in range(n_tokens):

@@ -138,6 +138,26 @@ def test_embed_swiglu_argmax(ctx):
         assert d_i.download(np.int32, 1)[0] == where, (n, where, shift)
 
 
+def test_greedy_next(ctx):
+    # the tail of a decode step in one launch: position + 1, arg-max, history, next embedding
+    V, H = 3000, 200
+    table = synth_normal(31, 1.0, (V, H))
+    d_table = ctx.to_device(table)
+    d_tok, d_hist, d_x = ctx.alloc(4), ctx.to_device(np.full(16, -1, np.int32)), ctx.alloc(4 * H)
+    d_pos = ctx.to_device(np.array([4], np.int32))
+    for step, where in enumerate((2999, 0, 1234)):
+        v = synth_normal(32 + step, 1.0, (V,))
+        v[where] = v.max() + 1
+        d_v = ctx.to_device(v)
+        check(ctx.lib.rbn_greedy_next_f32(ctx.handle, d_v.ptr, V, d_tok.ptr, d_hist.ptr, d_pos.ptr,
+                                          d_table.ptr, H, d_x.ptr))
+        assert d_tok.download(np.int32, 1)[0] == where
+        assert d_pos.download(np.int32, 1)[0] == 5 + step
+        assert d_hist.download(np.int32, 16)[5 + step] == where
+        assert (d_x.download(np.float32, H) == table[where]).all()
+    assert (d_hist.download(np.int32, 16)[:5] == -1).all()
+
+
 @pytest.mark.parametrize("M,pos0,heads", [(1, 0, 2), (1, 130, 3), (6, 0, 2), (5, 250, 2), (1, 1023, 1),
                                           (32, 0, 1), (64, 0, 2), (100, 37, 3), (33, 990, 1), (512, 0, 2),
                                           (200, 300, 1)])

@@ -30,7 +30,7 @@ INT8_PEAK_TOPS = 5000.0     # MI355X published dense int8 MFMA rate (5.0 POP/s)
 MALL_BYTES = 256 << 20
 # HBM bytes per launch of the headline GEMV, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a
 # 256 MiB copy (profiles/gemv_m1_k4096_n11008.md)
-GEMV_HEADLINE_TRAFFIC_BYTES = 11406785
+GEMV_HEADLINE_TRAFFIC_BYTES = 11406780
 
 
 def gemv_bytes(M, K, N):

@@ -290,6 +290,17 @@ def test_gemv_decode_sweep_shapes(ctx, M, K, N):
     check_against_oracle(x, w, *res, literal=(M == 1 and K * N <= 4096 * 4096))
 
 
+@pytest.mark.parametrize("M,K,N", [(1, 8192, 8452), (2, 8192, 8200), (1, 12288, 8200), (2, 15000, 260)])
+def test_gemv_long_rows(ctx, M, K, N):
+    # k long enough for eight (and more) 16-byte loads per lane: one round of eight in flight
+    # for K around 8192, rounds of four beyond; ragged N
+    say("gemv long rows", M, K, N)
+    x = synth_normal(0x5EED0041 + M, 1.0, (M, K))
+    w = synth_normal(0x5EED1041 + N, 0.015, (K, N))
+    res = run_matmul(ctx, ctx.gemv, x, w)
+    check_against_oracle(x, w, *res, literal=False)
+
+
 def test_gemv_reference_mode_config1(ctx):
     # the single-BitLinear configuration, x[1,2048] . W[2048,2048], both operands ternarised as the reference does
     x = synth_normal(0x5EED0001, 1.0, (1, 2048))

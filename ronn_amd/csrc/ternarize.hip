@@ -403,7 +403,14 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     __shared__ uint32_t s_cross_block, s_cross_k;
     __shared__ uint32_t s_bits_now;
     const uint32_t t = threadIdx.x;
-    if (state->done) {
+    // Windows of up to 1024 blocks (most of them) have one map per thread: it is requested
+    // here, before the state is known, so that the two round trips overlap (the buffer holds
+    // at least 1024 maps).
+    const SeqMap spec = maps[t];
+    const uint32_t done0 = state->done;
+    // (both values are named here so that both loads are issued before either is waited for)
+    asm volatile("" : : "v"(spec.d0), "v"(spec.d1), "s"(done0));
+    if (done0) {
         if (mirror && t == 0) *host_copy = *state;
         return;
     }
@@ -449,8 +456,12 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         auto walk_cached = [&](auto size_tag) {
             constexpr int C = decltype(size_tag)::value;
             SeqMap mm[C];
+            if constexpr (C == 1) {
+                mm[0] = spec;
+            } else {
 #pragma unroll
-            for (int i = 0; i < C; ++i) mm[i] = maps[lo + i < hi ? lo + i : (hi > 0 ? hi - 1 : 0)];
+                for (int i = 0; i < C; ++i) mm[i] = maps[lo + i < hi ? lo + i : (hi > 0 ? hi - 1 : 0)];
+            }
 #pragma unroll
             for (int i = 0; i < C; ++i)
                 if (lo + i < hi) mine = seq_compose(mine, mm[i]);
@@ -472,7 +483,9 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
                 }
             }
         };
-        if (chunk <= 8u) {
+        if (chunk == 1u) {
+            walk_cached(std::integral_constant<int, 1>{});
+        } else if (chunk <= 8u) {
             walk_cached(std::integral_constant<int, 8>{});
         } else if (chunk <= 32u) {
             walk_cached(std::integral_constant<int, 32>{});
@@ -725,11 +738,13 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     constexpr int kMapGrid = 8192;
     const uint64_t total_blocks = (n + kSeqTile - 1) / kSeqTile;
     void *ws = nullptr;
-    RBN_CHECK(rbn_workspace(ctx, kScratchHeader + total_blocks * sizeof(SeqMap) + kMapGrid * 8, &ws));
+    // at least 1024 map slots: the window-end kernel reads slot threadIdx.x before it knows the window
+    const uint64_t map_slots = total_blocks > 1024 ? total_blocks : 1024;
+    RBN_CHECK(rbn_workspace(ctx, kScratchHeader + map_slots * sizeof(SeqMap) + kMapGrid * 8, &ws));
     ReduceScratch *scr = (ReduceScratch *)ws;
     SeqMap *maps = (SeqMap *)((char *)ws + kScratchHeader);
     unsigned long long *count_parts =
-        d_packed ? (unsigned long long *)((char *)ws + kScratchHeader + total_blocks * sizeof(SeqMap)) : nullptr;
+        d_packed ? (unsigned long long *)((char *)ws + kScratchHeader + map_slots * sizeof(SeqMap)) : nullptr;
     if (d_packed) fill_u64_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(count_parts, kMapGrid);
     SeqState *h_state = (SeqState *)ctx->mailbox;
     memset(h_state, 0, sizeof(SeqState));

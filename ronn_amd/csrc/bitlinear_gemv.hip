@@ -72,6 +72,13 @@ __device__ __forceinline__ uint4 to_nibble_planes(uint4 a) {
     return p;
 }
 
+// Weights are read once per launch: non-temporal loads (see gemv.hip).
+__device__ __forceinline__ uint4 ld_w(const uint4 *p) {
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    const v4u v = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 // KS waves per column quad, L weight loads in flight per lane and round, SWIGLU input,
 // W waves per workgroup, NB blocks of 16 activations per thread (K <= 1024 * W * NB).
 template <int KS, int L, bool SWIGLU, int W, int NB>
@@ -135,7 +142,7 @@ __global__ __launch_bounds__(W * 64) void bitlinear_gemv_kernel(
 #pragma unroll
     for (int it = 0; it < L; ++it) {
         const int kb = sl_lo + it * 64 + lane;
-        w[it] = wq[kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)];
+        w[it] = ld_w(wq + (kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)));
     }
     // The residual the epilogue adds, requested behind the weights (one broadcast read per
     // wave) instead of at the very end, where its round trip would be exposed.
@@ -234,7 +241,7 @@ __global__ __launch_bounds__(W * 64) void bitlinear_gemv_kernel(
 #pragma unroll
         for (int it = 0; it < L; ++it) {
             const int kb = r0 + 64 * L + it * 64 + lane;
-            wn[it] = wq[kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)];
+            wn[it] = ld_w(wq + (kb < sl_hi ? kb : min(sl_lo + lane, KB - 1)));
         }
         consume(w, r0);
 #pragma unroll

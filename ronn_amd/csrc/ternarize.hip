@@ -13,6 +13,22 @@
 
 namespace {
 
+// NT: a non-temporal load, which keeps a streamed tensor from being allocated in the caches on
+// its way in.  It pays when the tensor is larger than the last-level cache (8192 x 28672 f32,
+// two tree passes: 0.41 -> 0.39 ms); a smaller one is still there for the second pass, and
+// the windows of the exact sequential sums re-read what they have just read.
+template <bool NT>
+__device__ __forceinline__ float4 ld_stream(const float4 *p) {
+    if constexpr (NT) {
+        typedef float v4f __attribute__((ext_vector_type(4)));
+        const v4f v = __builtin_nontemporal_load(reinterpret_cast<const v4f *>(p));
+        return make_float4(v.x, v.y, v.z, v.w);
+    } else {
+        return *p;
+    }
+}
+constexpr uint64_t kStreamBytes = 192ull << 20;  // tensors above this size are read non-temporally
+
 constexpr int kBlock = 256;
 constexpr int kSeqTile = 4096;  // elements per block map of the sequential sum (256 x 16)
 
@@ -28,6 +44,7 @@ __device__ __forceinline__ uint32_t ternary_code(float v, float threshold) {
 // every load instruction of a wave reads 1 KiB of consecutive floats.
 // `survivors` (optional) receives the number of elements with |x| > threshold.
 // ---------------------------------------------------------------------------
+template <bool NT>
 __global__ __launch_bounds__(kBlock) void pack_ternary_kernel(
     const float *__restrict__ x, uint64_t n, float threshold, uint32_t *__restrict__ packed,
     uint64_t n_tiles, unsigned long long *__restrict__ survivors, double *__restrict__ psum) {
@@ -45,7 +62,7 @@ __global__ __launch_bounds__(kBlock) void pack_ternary_kernel(
         for (int j = 0; j < 4; ++j) {
             uint64_t q = tile_quad0 + (uint64_t)j * kBlock + threadIdx.x;
             full[j] = (q * 4 + 3) < n;
-            v[j] = full[j] ? reinterpret_cast<const float4 *>(x)[q]
+            v[j] = full[j] ? ld_stream<NT>(reinterpret_cast<const float4 *>(x) + q)
                            : make_float4(0.f, 0.f, 0.f, 0.f);
         }
 #pragma unroll
@@ -131,6 +148,7 @@ __global__ __launch_bounds__(kBlock) void sum_partials_kernel(const double *__re
 // ---------------------------------------------------------------------------
 // Tree mode: deterministic f64 sum of |x| (optionally masked) and survivor count.
 // ---------------------------------------------------------------------------
+template <bool NT>
 __global__ __launch_bounds__(kBlock) void abs_sum_tree_partial_kernel(
     const float *__restrict__ x, uint64_t n, int use_mask, float thr, double *__restrict__ psum,
     unsigned long long *__restrict__ pcnt) {
@@ -154,7 +172,8 @@ __global__ __launch_bounds__(kBlock) void abs_sum_tree_partial_kernel(
         const uint64_t n4 = n / 4;
         uint64_t i = tid;
         for (; i + 3 * stride < n4; i += 4 * stride) {
-            const float4 a = x4[i], b = x4[i + stride], c = x4[i + 2 * stride], d = x4[i + 3 * stride];
+            const float4 a = ld_stream<NT>(x4 + i), b = ld_stream<NT>(x4 + i + stride),
+                         c = ld_stream<NT>(x4 + i + 2 * stride), d = ld_stream<NT>(x4 + i + 3 * stride);
             add(a.x), add(a.y), add(a.z), add(a.w);
             add(b.x), add(b.y), add(b.z), add(b.w);
             add(c.x), add(c.y), add(c.z), add(c.w);
@@ -828,8 +847,12 @@ int tree_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, float
     unsigned long long *pcnt = (unsigned long long *)(psum + kTreeParts);
     uint64_t want = (n + kSeqTile - 1) / kSeqTile;
     int parts = (int)(want < (uint64_t)kTreeParts ? want : (uint64_t)kTreeParts);
-    abs_sum_tree_partial_kernel<<<dim3(parts), dim3(kBlock), 0, ctx->stream>>>(d_x, n, use_mask,
-                                                                              thr, psum, pcnt);
+    if (n * 4 > kStreamBytes)
+        abs_sum_tree_partial_kernel<true><<<dim3(parts), dim3(kBlock), 0, ctx->stream>>>(d_x, n, use_mask,
+                                                                                        thr, psum, pcnt);
+    else
+        abs_sum_tree_partial_kernel<false><<<dim3(parts), dim3(kBlock), 0, ctx->stream>>>(d_x, n, use_mask,
+                                                                                         thr, psum, pcnt);
     abs_sum_tree_final_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(
         psum, pcnt, parts, &scr->tree_sum, &scr->tree_cnt);
     RBN_HIP(hipGetLastError());
@@ -868,8 +891,12 @@ int pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold, ui
     uint64_t tiles = (n + kSeqTile - 1) / kSeqTile;
     if (tiles > 0x7fffffffull) return rbn_fail(RBN_ERR_UNSUPPORTED, "tensor too large");
     const unsigned grid = (unsigned)(tiles < (uint64_t)kPackGrid ? tiles : (uint64_t)kPackGrid);
-    pack_ternary_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
-        d_x, n, threshold, (uint32_t *)d_packed, tiles, d_cnt, d_psum);
+    if (n * 4 > kStreamBytes)
+        pack_ternary_kernel<true><<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
+            d_x, n, threshold, (uint32_t *)d_packed, tiles, d_cnt, d_psum);
+    else
+        pack_ternary_kernel<false><<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
+            d_x, n, threshold, (uint32_t *)d_packed, tiles, d_cnt, d_psum);
     if (d_psum)
         sum_partials_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(d_psum, (int)grid, &scr->tree_sum);
     RBN_HIP(hipGetLastError());

@@ -521,11 +521,18 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
         const int t0 = b * 16, last = max(nkeys - 1 - t0, 0);
         const int t = t0 + min(kidx, last);
         const uint4 *krow = reinterpret_cast<const uint4 *>(kh + (size_t)t * hd + sub * 32);
+        typedef unsigned v4u __attribute__((ext_vector_type(4)));
 #pragma unroll
-        for (int c = 0; c < 4; ++c) kr[c] = krow[c];
+        for (int c = 0; c < 4; ++c) {
+            const v4u kv = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(krow + c));
+            kr[c] = make_uint4(kv.x, kv.y, kv.z, kv.w);
+        }
 #pragma unroll
-        for (int j = 0; j < 16; ++j)
-            vr[j] = *reinterpret_cast<const __half2 *>(vh + (size_t)(t0 + min(j, last)) * hd + 2 * lane);
+        for (int j = 0; j < 16; ++j) {
+            const unsigned vv = __builtin_nontemporal_load(
+                reinterpret_cast<const unsigned *>(vh + (size_t)(t0 + min(j, last)) * hd + 2 * lane));
+            vr[j] = *reinterpret_cast<const __half2 *>(&vv);
+        }
     };
     int b = sp * 4 + wave;
     bool have = b * 16 < nkeys;

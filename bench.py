@@ -30,7 +30,7 @@ INT8_PEAK_TOPS = 5000.0     # MI355X published dense int8 MFMA rate (5.0 POP/s)
 MALL_BYTES = 256 << 20
 # HBM bytes per launch of the headline GEMV, from rocprofv3 FETCH_SIZE + WRITE_SIZE scaled by a
 # 256 MiB copy (profiles/gemv_m1_k4096_n11008.md)
-GEMV_HEADLINE_TRAFFIC_BYTES = 11406780
+GEMV_HEADLINE_TRAFFIC_BYTES = 11415105
 
 
 def gemv_bytes(M, K, N):
@@ -342,6 +342,20 @@ def main():
                                     "GBps": bytes_per_launch / (ev1 * 1e-3) / 1e9,
                                     "note": "single 11 MiB weight buffer re-read from cache, not HBM"}
         del one
+        # One launch at a time on an idle stream, timed by the dispatch's own begin and end
+        # timestamps: what a profiler's kernel trace reports.  Back to back (the timed region
+        # above) a launch starts while the one before it drains, so a step is shorter than this.
+        iso = Workload(ctx, M, K, N, 0.02, seed=2, mode=1)  # default rotation: more than the Infinity Cache
+        iso_us = []
+        for i in range(130):
+            j = i % len(iso.tiled)
+            iso_us.append(ctx.gemv_kernel_time_us(iso.acts, iso.tiled[j], iso.w_scale, M, K, N, iso.d_out))
+        iso_us = sorted(iso_us[30:])
+        extra["gemv_isolated_dispatch"] = {"us_mean": sum(iso_us) / len(iso_us), "us_median": iso_us[len(iso_us) // 2],
+                                           "us_min": iso_us[0],
+                                           "note": "begin-to-end timestamps of single dispatches on an idle stream "
+                                                   "(rbn_gemv_t2_i8_kernel_time); compare rocprofv3's kernel trace"}
+        del iso
         def kernel_for(m, k, n):
             return ("gemv", "skinny_mfma", "gemm_mfma")[ctx.lib.rbn_matmul_kernel_choice(m, k, n)]
 

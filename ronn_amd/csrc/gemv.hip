@@ -26,6 +26,7 @@
 //    per-token sum of q is subtracted once in the epilogue.  All of it is
 //    integer-exact.
 #include "common.hpp"
+#include <hip/hip_ext.h>
 
 namespace {
 
@@ -277,6 +278,7 @@ struct Args {
     const uint4 *w4;
     float w_scale;
     int M, KB, KC, N, nquads, vec_store, exact;
+    hipEvent_t ev_begin = nullptr, ev_end = nullptr;
     int32_t *acc;
     float *out;
 };
@@ -286,16 +288,23 @@ void launch(hipStream_t stream, const Args &a) {
     constexpr int QPB = kWaves / KS;
     dim3 grid((unsigned)((a.nquads + QPB - 1) / QPB));
     const size_t lds = (size_t)MT * a.KC * 16;
+    // with events given the launch records the kernel's own begin and end timestamps in them
+    auto go = [&](auto kernel) {
+        if (a.ev_begin)
+            hipExtLaunchKernelGGL(kernel, grid, dim3(kThreads), lds, stream, a.ev_begin, a.ev_end, 0, a.q4,
+                                  a.act_scale, a.rowsum, a.w4, a.w_scale, a.M, a.KB, a.KC, a.N, a.nquads,
+                                  a.vec_store, a.acc, a.out);
+        else
+            kernel<<<grid, dim3(kThreads), lds, stream>>>(a.q4, a.act_scale, a.rowsum, a.w4, a.w_scale, a.M,
+                                                         a.KB, a.KC, a.N, a.nquads, a.vec_store, a.acc, a.out);
+    };
     if constexpr (KS == 1 && MT <= 4) {
         if (a.exact && a.KC == a.KB && a.KB % (64 * L) == 0) {
-            gemv_t2_i8_kernel<MT, KS, L, true><<<grid, dim3(kThreads), lds, stream>>>(
-                a.q4, a.act_scale, a.rowsum, a.w4, a.w_scale, a.M, a.KB, a.KC, a.N, a.nquads, a.vec_store, a.acc,
-                a.out);
+            go(gemv_t2_i8_kernel<MT, KS, L, true>);
             return;
         }
     }
-    gemv_t2_i8_kernel<MT, KS, L, false><<<grid, dim3(kThreads), lds, stream>>>(
-        a.q4, a.act_scale, a.rowsum, a.w4, a.w_scale, a.M, a.KB, a.KC, a.N, a.nquads, a.vec_store, a.acc, a.out);
+    go(gemv_t2_i8_kernel<MT, KS, L, false>);
 }
 
 template <int MT, int KS>
@@ -331,9 +340,9 @@ void launch_ks(hipStream_t stream, const Args &a, int ks) {
 
 }  // namespace
 
-extern "C" int rbn_gemv_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
-                              const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
-                              uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out) {
+static int gemv_impl(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale, const int32_t *d_rowsum,
+                     const uint32_t *d_tiled, float w_scale, uint64_t M, uint64_t K, uint64_t N,
+                     int32_t *d_acc, float *d_out, float *h_kernel_us) {
     RBN_ENTER(ctx);
     RBN_REQUIRE(M > 0 && K > 0 && N > 0, "M, K and N must be positive");
     RBN_REQUIRE(M <= RBN_GEMV_MAX_M, "rbn_gemv_t2_i8 takes M <= %d (got %llu)", RBN_GEMV_MAX_M,
@@ -354,6 +363,10 @@ extern "C" int rbn_gemv_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_ac
     a.nquads = (int)(rbn_npad(N) / 4);
     a.acc = d_acc;
     a.out = d_out;
+    if (h_kernel_us) {
+        a.ev_begin = ctx->ev_start;
+        a.ev_end = ctx->ev_stop;
+    }
     a.vec_store = N % 4 == 0 && (((uintptr_t)d_out | (uintptr_t)d_acc) & 15u) == 0;
     a.exact = 1;
     const int mt = M == 1 ? 1 : M == 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
@@ -380,5 +393,28 @@ extern "C" int rbn_gemv_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_ac
         default: launch_ks<16>(ctx->stream, a, ks); break;
     }
     RBN_HIP(hipGetLastError());
+    if (h_kernel_us) {
+        float ms = 0.0f;
+        RBN_HIP(hipEventSynchronize(ctx->ev_stop));
+        RBN_HIP(hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop));
+        *h_kernel_us = ms * 1000.0f;
+    }
     return RBN_OK;
+}
+
+extern "C" int rbn_gemv_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
+                              const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
+                              uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out) {
+    return gemv_impl(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N, d_acc, d_out, nullptr);
+}
+
+extern "C" int rbn_gemv_t2_i8_kernel_time(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
+                                          const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
+                                          uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out,
+                                          float *h_kernel_us) {
+    if (ctx && !h_kernel_us) {
+        RBN_ENTER(ctx);
+        return rbn_fail(RBN_ERR_INVALID, "h_kernel_us is NULL");
+    }
+    return gemv_impl(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N, d_acc, d_out, h_kernel_us);
 }

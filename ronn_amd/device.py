@@ -207,6 +207,14 @@ class Context:
         return self._mm(self.lib.rbn_gemv_t2_i8, acts, d_tiled, w_scale, M, K, N, want_acc, d_out,
                         d_acc)
 
+    def gemv_kernel_time_us(self, acts, d_tiled, w_scale, M, K, N, d_out) -> float:
+        """One GEMV launch; returns the duration of the dispatch from its own timestamps."""
+        d_q, d_s, d_r = acts
+        us = C.c_float()
+        check(self.lib.rbn_gemv_t2_i8_kernel_time(self.handle, d_q.ptr, d_s.ptr, d_r.ptr, d_tiled.ptr,
+                                                  float(w_scale), M, K, N, None, d_out.ptr, C.byref(us)))
+        return us.value
+
     def skinny(self, acts, d_tiled, w_scale, M, K, N, want_acc=False, d_out=None, d_acc=None):
         return self._mm(self.lib.rbn_gemm_t2_i8_skinny, acts, d_tiled, w_scale, M, K, N, want_acc,
                         d_out, d_acc)

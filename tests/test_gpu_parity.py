@@ -301,6 +301,22 @@ def test_gemv_long_rows(ctx, M, K, N):
     check_against_oracle(x, w, *res, literal=False)
 
 
+def test_gemv_kernel_time_entry(ctx):
+    # the measuring variant launches the same kernel and reports the dispatch's own duration
+    M, K, N = 1, 2048, 1024
+    x = synth_normal(0x5EED0051, 1.0, (M, K))
+    w = synth_normal(0x5EED1051, 0.02, (K, N))
+    ref = run_matmul(ctx, ctx.gemv, x, w)
+    d_w = ctx.to_device(w)
+    d_p, w_scale, _, _ = ctx.quantize_ternary(d_w, K * N, _lib.SUM_STRICT_SEQ)
+    tiled = ctx.tile_weights(d_p, K, N)
+    acts = ctx.act_quant_i8(ctx.to_device(x), M, K)
+    d_out = ctx.alloc(4 * M * N)
+    us = ctx.gemv_kernel_time_us(acts, tiled, w_scale, M, K, N, d_out)
+    assert 0.5 < us < 1000.0
+    assert same_bits(d_out.download(np.float32, M * N).reshape(M, N), ref[0])
+
+
 def test_gemv_reference_mode_config1(ctx):
     # the single-BitLinear configuration, x[1,2048] . W[2048,2048], both operands ternarised as the reference does
     x = synth_normal(0x5EED0001, 1.0, (1, 2048))

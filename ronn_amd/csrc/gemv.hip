@@ -277,7 +277,7 @@ struct Args {
     const int32_t *rowsum;
     const uint4 *w4;
     float w_scale;
-    int M, KB, KC, N, nquads, vec_store, exact;
+    int M, KB, KC, N, nquads, vec_store;
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
     int32_t *acc;
     float *out;
@@ -299,7 +299,7 @@ void launch(hipStream_t stream, const Args &a) {
                                                          a.KB, a.KC, a.N, a.nquads, a.vec_store, a.acc, a.out);
     };
     if constexpr (KS == 1 && MT <= 4) {
-        if (a.exact && a.KC == a.KB && a.KB % (64 * L) == 0) {
+        if (a.KC == a.KB && a.KB % (64 * L) == 0) {
             go(gemv_t2_i8_kernel<MT, KS, L, true>);
             return;
         }
@@ -368,7 +368,6 @@ static int gemv_impl(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale, 
         a.ev_end = ctx->ev_stop;
     }
     a.vec_store = N % 4 == 0 && (((uintptr_t)d_out | (uintptr_t)d_acc) & 15u) == 0;
-    a.exact = 1;
     const int mt = M == 1 ? 1 : M == 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
     // k-blocks whose staged activations fit the LDS budget in one pass
     const int kc_cap = kLdsBudget / 16 / mt;

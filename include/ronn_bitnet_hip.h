@@ -203,7 +203,9 @@ int rbn_gemv_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
                    uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);
 /* rbn_gemv_t2_i8, launched so that the kernel's own begin and end timestamps are recorded:
  * *h_kernel_us receives the duration of this one dispatch (what a profiler's kernel trace
- * reports).  Synchronises the stream.  For measurement; no counterpart in the reference. */
+ * reports).  Synchronises the stream and uses the context's timer events, so it must not sit
+ * between rbn_timer_start and rbn_timer_stop, nor inside a graph capture.  For measurement;
+ * no counterpart in the reference. */
 int rbn_gemv_t2_i8_kernel_time(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
                                const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
                                uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out,

@@ -156,6 +156,13 @@ def test_greedy_next(ctx):
         assert d_hist.download(np.int32, 16)[5 + step] == where
         assert (d_x.download(np.float32, H) == table[where]).all()
     assert (d_hist.download(np.int32, 16)[:5] == -1).all()
+    # null pointers and empty sizes are refused, not launched
+    for args in ((None, V, d_tok.ptr, d_hist.ptr, d_pos.ptr, d_table.ptr, H, d_x.ptr),
+                 (d_v.ptr, 0, d_tok.ptr, d_hist.ptr, d_pos.ptr, d_table.ptr, H, d_x.ptr),
+                 (d_v.ptr, V, d_tok.ptr, d_hist.ptr, d_pos.ptr, None, H, d_x.ptr)):
+        with pytest.raises(_lib.RbnError) as e:
+            check(ctx.lib.rbn_greedy_next_f32(ctx.handle, *args))
+        assert e.value.code == _lib.RBN_ERR_INVALID
 
 
 @pytest.mark.parametrize("M,pos0,heads", [(1, 0, 2), (1, 130, 3), (6, 0, 2), (5, 250, 2), (1, 1023, 1),

@@ -379,10 +379,10 @@ static int gemv_impl(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale, 
     if (M == 1) {
         if (a.nquads <= 1024 && a.KB >= 640)
             ks = 4;
-        else if ((a.nquads <= 1024 && a.KB >= 160) || (a.nquads <= 2048 && a.KB >= 512))
+        else if (a.nquads <= 1024 && a.KB >= 320)
             ks = 2;
     } else {
-        while (ks < 4 && (long long)a.nquads * ks < 2048 && a.KB / (ks * 2) >= 128) ks *= 2;
+        while (ks < 4 && (long long)a.nquads * ks < 2048 && a.KB / (ks * 2) >= 160) ks *= 2;
     }
     switch (mt) {
         case 1: launch_ks<1>(ctx->stream, a, ks); break;

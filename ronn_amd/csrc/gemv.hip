@@ -382,7 +382,10 @@ static int gemv_impl(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale, 
         else if (a.nquads <= 1024 && a.KB >= 320)
             ks = 2;
     } else {
-        while (ks < 4 && (long long)a.nquads * ks < 2048 && a.KB / (ks * 2) >= 160) ks *= 2;
+        // (a share of 128-159 k-blocks only when the waves would otherwise be few)
+        while (ks < 4 && (long long)a.nquads * ks < 2048 &&
+               (a.KB / (ks * 2) >= 160 || (a.KB / (ks * 2) >= 128 && (long long)a.nquads * ks < 1024)))
+            ks *= 2;
     }
     switch (mt) {
         case 1: launch_ks<1>(ctx->stream, a, ks); break;

@@ -99,6 +99,11 @@ int rbn_d2h(rbn_ctx *ctx, void *h_dst, const void *d_src, size_t bytes);
 int rbn_d2d(rbn_ctx *ctx, void *d_dst, const void *d_src, size_t bytes);
 int rbn_fill_u8(rbn_ctx *ctx, void *d_dst, int value, size_t bytes);
 int rbn_sync(rbn_ctx *ctx);
+/* Conditions that only a kernel can see are reported through one word of flags per
+ * context: *h_flags receives the bits raised since the last call and the word is cleared.
+ * Synchronises the stream.  No reference counterpart. */
+#define RBN_FLAG_HISTORY_OVERFLOW 1u /* rbn_argmax_f32 / rbn_greedy_next_f32: position outside the history */
+int rbn_device_flags(rbn_ctx *ctx, uint32_t *h_flags);
 /* Bytes currently / at most allocated through rbn_malloc on this context
  * (MemoryInfo, allocator.rs:142-148). */
 int rbn_memory_info(rbn_ctx *ctx, uint64_t *allocated, uint64_t *peak);
@@ -279,16 +284,22 @@ int rbn_attention_decode_f16kv(rbn_ctx *ctx, const float *d_qkv, const int32_t *
 /* h[m,f] = silu(gu[m,f]) * gu[m,F+f], gu [M, 2F]. */
 int rbn_swiglu_f32(rbn_ctx *ctx, const float *d_gate_up, uint64_t M, uint64_t F, float *d_h);
 /* *d_index = index of the largest value (lowest index among equals).  If d_history
- * is given the index is also written to d_history[*d_history_pos]. */
+ * (history_capacity int32 entries) is given the index is also written to
+ * d_history[*d_history_pos]; a position outside [0, history_capacity) writes nothing and
+ * raises RBN_FLAG_HISTORY_OVERFLOW (rbn_device_flags). */
 int rbn_argmax_f32(rbn_ctx *ctx, const float *d_values, uint64_t n, int32_t *d_index,
-                   int32_t *d_history, const int32_t *d_history_pos);
+                   int32_t *d_history, const int32_t *d_history_pos, uint64_t history_capacity);
 /* The tail of a greedy decode step in one launch: *d_pos += 1; t = arg-max of the vocab
  * logits (lowest index among equals); *d_token = t; d_history[*d_pos] = t; d_x[0..H) =
- * d_table[t, :] (the next step's embedding).  No counterpart in the reference (decoder
- * harness). */
+ * d_table[t, :] (the next step's embedding).  d_history holds history_capacity entries:
+ * when *d_pos + 1 would leave it, the position stays, nothing is written to the history
+ * and RBN_FLAG_HISTORY_OVERFLOW is raised (*d_token and d_x are still written).  The
+ * attention kernels clamp positions to max_seq - 1 on their own: past the end of the K/V
+ * cache they overwrite its last row and the output is meaningless, so a caller has to
+ * stop at the capacity.  No counterpart in the reference (decoder harness). */
 int rbn_greedy_next_f32(rbn_ctx *ctx, const float *d_logits, uint64_t vocab, int32_t *d_token,
-                        int32_t *d_history, int32_t *d_pos, const float *d_table, uint64_t H,
-                        float *d_x);
+                        int32_t *d_history, int32_t *d_pos, uint64_t history_capacity,
+                        const float *d_table, uint64_t H, float *d_x);
 /* *d_value += delta (the position counter of a captured decode step). */
 int rbn_add_i32(rbn_ctx *ctx, int32_t *d_value, int32_t delta);
 /* Normal(0, sigma) values generated on the device (counter-based, f32 Box-Muller);

@@ -22,6 +22,7 @@ RBN_ERR_NO_DEVICE = -5
 SUM_STRICT_SEQ = 0
 SUM_TREE = 1
 GEMV_MAX_M = 16
+FLAG_HISTORY_OVERFLOW = 1
 
 # dtype codes of rbn_tensor_bytes (declaration order of the reference's DataType)
 DT_F32, DT_F16, DT_BF16, DT_I8, DT_I32, DT_I64, DT_U8, DT_U32, DT_BOOL, DT_F64 = range(10)
@@ -99,8 +100,9 @@ SIGNATURES = {
     "rbn_attention_f16kv": (C.c_int, [_vp, _vp, _vp, _u64, _u64, _u64, _vp, _vp, _u64, _vp]),
     "rbn_attention_decode_f16kv": (C.c_int, [_vp, _vp, _vp, _u64, _u64, C.c_float, _vp, _vp, _u64, _vp]),
     "rbn_swiglu_f32": (C.c_int, [_vp, _vp, _u64, _u64, _vp]),
-    "rbn_argmax_f32": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _vp]),
-    "rbn_greedy_next_f32": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _vp, _vp, _u64, _vp]),
+    "rbn_argmax_f32": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _vp, _u64]),
+    "rbn_greedy_next_f32": (C.c_int, [_vp, _vp, _u64, _vp, _vp, _vp, _u64, _vp, _u64, _vp]),
+    "rbn_device_flags": (C.c_int, [_vp, C.POINTER(C.c_uint32)]),
     "rbn_add_i32": (C.c_int, [_vp, _vp, C.c_int32]),
     "rbn_synth_normal_device_f32": (C.c_int, [_vp, _u64, C.c_float, _vp, _u64]),
     "rbn_probe_mfma_i8": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_double)]),

@@ -31,6 +31,9 @@ struct rbn_ctx {
     // context and never moved, so launches captured in a HIP graph stay valid.
     void *splitk_partials = nullptr;
     unsigned *splitk_tickets = nullptr;
+    // One word of RBN_FLAG_* bits that kernels set when they refuse to do something a host
+    // check could not see coming (rbn_device_flags reads and clears it).
+    unsigned *dev_flags = nullptr;
 };
 
 constexpr int RBN_SPLITK_TILES = 16384;  // 64 MiB

@@ -94,7 +94,9 @@ int rbn_ctx_create(int device, rbn_ctx **out) {
         (e = hipHostMalloc(&ctx->mailbox, 4096, hipHostMallocDefault)) != hipSuccess ||
         (e = hipMalloc(&ctx->splitk_partials, (size_t)RBN_SPLITK_TILES * 4096)) != hipSuccess ||
         (e = hipMalloc((void **)&ctx->splitk_tickets, RBN_SPLITK_GROUPS * sizeof(unsigned))) != hipSuccess ||
-        (e = hipMemset(ctx->splitk_tickets, 0, RBN_SPLITK_GROUPS * sizeof(unsigned))) != hipSuccess) {
+        (e = hipMemset(ctx->splitk_tickets, 0, RBN_SPLITK_GROUPS * sizeof(unsigned))) != hipSuccess ||
+        (e = hipMalloc((void **)&ctx->dev_flags, 256)) != hipSuccess ||
+        (e = hipMemset(ctx->dev_flags, 0, 256)) != hipSuccess) {
         int rc = rbn_fail(RBN_ERR_HIP, "context set-up failed: %s", hipGetErrorString(e));
         rbn_ctx_destroy(ctx);
         return rc;
@@ -116,6 +118,7 @@ int rbn_ctx_destroy(rbn_ctx *ctx) {
     if (ctx->mailbox) (void)hipHostFree(ctx->mailbox);
     if (ctx->splitk_partials) (void)hipFree(ctx->splitk_partials);
     if (ctx->splitk_tickets) (void)hipFree(ctx->splitk_tickets);
+    if (ctx->dev_flags) (void)hipFree(ctx->dev_flags);
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
     if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
@@ -207,6 +210,18 @@ int rbn_fill_u8(rbn_ctx *ctx, void *d_dst, int value, size_t bytes) {
 int rbn_sync(rbn_ctx *ctx) {
     RBN_ENTER(ctx);
     RBN_HIP(hipStreamSynchronize(ctx->stream));
+    return RBN_OK;
+}
+
+int rbn_device_flags(rbn_ctx *ctx, uint32_t *h_flags) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(h_flags != nullptr, "h_flags is NULL");
+    unsigned *box = static_cast<unsigned *>(ctx->mailbox) + 512;  // the mailbox's second half
+    RBN_HIP(hipMemcpyAsync(box, ctx->dev_flags, sizeof(unsigned), hipMemcpyDeviceToHost, ctx->stream));
+    fill_u8_kernel<<<dim3(1), dim3(64), 0, ctx->stream>>>((uint8_t *)ctx->dev_flags, 0, sizeof(unsigned));
+    RBN_HIP(hipGetLastError());
+    RBN_HIP(hipStreamSynchronize(ctx->stream));
+    *h_flags = *box;
     return RBN_OK;
 }
 

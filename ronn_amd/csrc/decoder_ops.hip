@@ -670,12 +670,13 @@ __global__ __launch_bounds__(kBlock) void swiglu_kernel(const float *__restrict_
 
 // Index of the largest of n values (the lowest index among equals); one workgroup.
 // With `advance` the position counter hist_pos[0] is incremented first (the history slot is
-// the new position); with `table` the row of the chosen index is copied to x_out (the next
+// the new position); the history holds hist_cap entries; with `table` the row of the chosen index is copied to x_out (the next
 // step's embedding): the tail of a greedy decode step in one launch.
 __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ v, int n,
                                                       int32_t *__restrict__ out,
                                                       int32_t *__restrict__ hist,
-                                                      int32_t *__restrict__ hist_pos, int advance,
+                                                      int32_t *__restrict__ hist_pos, int hist_cap,
+                                                      unsigned *__restrict__ dev_flags, int advance,
                                                       const float *__restrict__ table, int H,
                                                       float *__restrict__ x_out) {
     __shared__ float s_v[16];
@@ -732,9 +733,15 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
         bi = bi == 0x7fffffff ? 0 : bi;
         out[0] = bi;
         if (hist) {
-            int p = hist_pos[0];
-            if (advance) hist_pos[0] = ++p;
-            hist[p] = bi;
+            // a slot outside the history is neither written nor made the new position; the
+            // host learns of it through the context's flag word
+            const int p = hist_pos[0] + (advance ? 1 : 0);
+            if (p >= 0 && p < hist_cap) {
+                if (advance) hist_pos[0] = p;
+                hist[p] = bi;
+            } else {
+                atomicOr(dev_flags, (unsigned)RBN_FLAG_HISTORY_OVERFLOW);
+            }
         }
         s_pick = bi;
     }
@@ -872,28 +879,34 @@ int rbn_swiglu_f32(rbn_ctx *ctx, const float *d_gate_up, uint64_t M, uint64_t F,
 }
 
 int rbn_argmax_f32(rbn_ctx *ctx, const float *d_values, uint64_t n, int32_t *d_index,
-                   int32_t *d_history, const int32_t *d_history_pos) {
+                   int32_t *d_history, const int32_t *d_history_pos, uint64_t history_capacity) {
     RBN_ENTER(ctx);
     RBN_REQUIRE(d_values && d_index, "null pointer in rbn_argmax_f32");
     RBN_REQUIRE(n > 0 && n < (1u << 30), "bad n in rbn_argmax_f32");
     RBN_REQUIRE((d_history == nullptr) == (d_history_pos == nullptr),
                 "d_history and d_history_pos go together");
+    RBN_REQUIRE(d_history == nullptr || (history_capacity > 0 && history_capacity < (1ull << 31)),
+                "history_capacity must be in [1, 2^31) when d_history is given");
     argmax_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(d_values, (int)n, d_index, d_history,
-                                                          const_cast<int32_t *>(d_history_pos), 0, nullptr,
+                                                          const_cast<int32_t *>(d_history_pos),
+                                                          (int)history_capacity, ctx->dev_flags, 0, nullptr,
                                                           0, nullptr);
     RBN_HIP(hipGetLastError());
     return RBN_OK;
 }
 
 int rbn_greedy_next_f32(rbn_ctx *ctx, const float *d_logits, uint64_t vocab, int32_t *d_token,
-                        int32_t *d_history, int32_t *d_pos, const float *d_table, uint64_t H,
-                        float *d_x) {
+                        int32_t *d_history, int32_t *d_pos, uint64_t history_capacity,
+                        const float *d_table, uint64_t H, float *d_x) {
     RBN_ENTER(ctx);
     RBN_REQUIRE(d_logits && d_token && d_history && d_pos && d_table && d_x && vocab > 0 && H > 0 &&
                     vocab < (1ull << 31) && H < (1ull << 31),
                 "bad arguments in rbn_greedy_next_f32");
+    RBN_REQUIRE(history_capacity > 0 && history_capacity < (1ull << 31),
+                "history_capacity must be in [1, 2^31)");
     argmax_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(d_logits, (int)vocab, d_token, d_history, d_pos,
-                                                          1, d_table, (int)H, d_x);
+                                                          (int)history_capacity, ctx->dev_flags, 1, d_table,
+                                                          (int)H, d_x);
     RBN_HIP(hipGetLastError());
     return RBN_OK;
 }

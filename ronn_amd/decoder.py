@@ -81,6 +81,7 @@ class BitNetDecoder:
         self.blocks = []
         self.embed = self.g_final = self.lm_head = None
         self._graph = None
+        self._pos = 0   # host copy of the device position counter
 
     # -- weights ---------------------------------------------------------------------------
     def _linear_from_device_f32(self, d_w: DeviceBuffer, K: int, N: int) -> _Linear:
@@ -187,7 +188,7 @@ class BitNetDecoder:
         self._bitlinear1(self.lm_head, self.g_final, self.logits, x=self.x)
         # position + 1, arg-max, history, and the next step's embedding in one launch
         check(lib.rbn_greedy_next_f32(hnd, self.logits.ptr, cfg.vocab, self.tokens.ptr, self.history.ptr,
-                                      self.pos.ptr, self.embed.ptr, cfg.hidden, self.x.ptr))
+                                      self.pos.ptr, cfg.max_seq, self.embed.ptr, cfg.hidden, self.x.ptr))
 
     def forward(self, M: int):
         """Tokens self.tokens[0:M] at positions *pos .. *pos+M-1; leaves the logits of the
@@ -227,17 +228,26 @@ class BitNetDecoder:
         self._linear(self.lm_head, 1, self.logits)
         check(lib.rbn_add_i32(hnd, self.pos.ptr, M))
         check(lib.rbn_argmax_f32(hnd, self.logits.ptr, cfg.vocab, self.tokens.ptr, self.history.ptr,
-                                 self.pos.ptr))
+                                 self.pos.ptr, cfg.max_seq))
 
     # -- generation ------------------------------------------------------------------------
     def reset(self):
         check(self.lib.rbn_fill_u8(self.ctx.handle, self.pos.ptr, 0, 4))
+        self._pos = 0
 
     def prefill(self, prompt: np.ndarray):
+        """Runs the prompt from position 0.  The token predicted after it goes to history slot
+        len(prompt), so the prompt has to be shorter than max_seq."""
         prompt = np.ascontiguousarray(prompt, dtype=np.int32)
+        if prompt.ndim != 1 or len(prompt) == 0:
+            raise ValueError("the prompt must be a non-empty vector of token ids")
+        if len(prompt) >= self.cfg.max_seq:
+            raise ValueError("a prompt of %d tokens does not fit max_seq = %d (history slot %d is needed)"
+                             % (len(prompt), self.cfg.max_seq, len(prompt)))
         self.reset()
         check(self.lib.rbn_h2d(self.ctx.handle, self.tokens.ptr, prompt.ctypes.data, prompt.nbytes))
         self.forward(len(prompt))
+        self._pos = len(prompt)
 
     def capture_decode_step(self):
         if self._graph is None:
@@ -248,6 +258,9 @@ class BitNetDecoder:
 
     def decode(self, n_tokens: int, use_graph: bool = True):
         """Greedy decoding of n_tokens more tokens; returns (tokens, seconds)."""
+        if n_tokens < 0 or self._pos + n_tokens >= self.cfg.max_seq:
+            raise ValueError("decoding %d tokens from position %d would pass max_seq = %d"
+                             % (n_tokens, self._pos, self.cfg.max_seq))
         g = self.capture_decode_step() if use_graph else None
         # a step expects the embedding of the previous token in self.x (each step leaves the
         # next one's there; after a prompt it has to be looked up once)
@@ -262,6 +275,7 @@ class BitNetDecoder:
                 self.forward_one()
         self.ctx.sync()
         dt = time.perf_counter() - t0
+        self._pos += n_tokens
         return self.generated(n_tokens + 1)[1:], dt
 
     def generated(self, n: int) -> np.ndarray:

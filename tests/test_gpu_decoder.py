@@ -124,7 +124,7 @@ def test_embed_swiglu_argmax(ctx):
     v = synth_normal(23, 1.0, (32000,))
     v[77] = v[31000] = v.max() + 1                                       # a tie: lowest index wins
     d_i, d_hist, d_pos, d_v = ctx.alloc(4), ctx.alloc(64), ctx.to_device(np.array([3], np.int32)), ctx.to_device(v)
-    check(ctx.lib.rbn_argmax_f32(ctx.handle, d_v.ptr, v.size, d_i.ptr, d_hist.ptr, d_pos.ptr))
+    check(ctx.lib.rbn_argmax_f32(ctx.handle, d_v.ptr, v.size, d_i.ptr, d_hist.ptr, d_pos.ptr, 16))
     assert d_i.download(np.int32, 1)[0] == 77 and d_hist.download(np.int32, 16)[3] == 77
     check(ctx.lib.rbn_add_i32(ctx.handle, d_pos.ptr, 5))
     assert d_pos.download(np.int32, 1)[0] == 8
@@ -134,7 +134,7 @@ def test_embed_swiglu_argmax(ctx):
         w = synth_normal(24 + n, 1.0, (n + shift,))
         w[shift + where] = w.max() + 1
         d_w = ctx.to_device(w)
-        check(ctx.lib.rbn_argmax_f32(ctx.handle, d_w.ptr + 4 * shift, n, d_i.ptr, None, None))
+        check(ctx.lib.rbn_argmax_f32(ctx.handle, d_w.ptr + 4 * shift, n, d_i.ptr, None, None, 0))
         assert d_i.download(np.int32, 1)[0] == where, (n, where, shift)
 
 
@@ -149,7 +149,7 @@ def test_greedy_next(ctx):
         v = synth_normal(32 + step, 1.0, (V,))
         v[where] = v.max() + 1
         d_v = ctx.to_device(v)
-        check(ctx.lib.rbn_greedy_next_f32(ctx.handle, d_v.ptr, V, d_tok.ptr, d_hist.ptr, d_pos.ptr,
+        check(ctx.lib.rbn_greedy_next_f32(ctx.handle, d_v.ptr, V, d_tok.ptr, d_hist.ptr, d_pos.ptr, 16,
                                           d_table.ptr, H, d_x.ptr))
         assert d_tok.download(np.int32, 1)[0] == where
         assert d_pos.download(np.int32, 1)[0] == 5 + step
@@ -157,12 +157,71 @@ def test_greedy_next(ctx):
         assert (d_x.download(np.float32, H) == table[where]).all()
     assert (d_hist.download(np.int32, 16)[:5] == -1).all()
     # null pointers and empty sizes are refused, not launched
-    for args in ((None, V, d_tok.ptr, d_hist.ptr, d_pos.ptr, d_table.ptr, H, d_x.ptr),
-                 (d_v.ptr, 0, d_tok.ptr, d_hist.ptr, d_pos.ptr, d_table.ptr, H, d_x.ptr),
-                 (d_v.ptr, V, d_tok.ptr, d_hist.ptr, d_pos.ptr, None, H, d_x.ptr)):
+    for args in ((None, V, d_tok.ptr, d_hist.ptr, d_pos.ptr, 16, d_table.ptr, H, d_x.ptr),
+                 (d_v.ptr, 0, d_tok.ptr, d_hist.ptr, d_pos.ptr, 16, d_table.ptr, H, d_x.ptr),
+                 (d_v.ptr, V, d_tok.ptr, d_hist.ptr, d_pos.ptr, 0, d_table.ptr, H, d_x.ptr),
+                 (d_v.ptr, V, d_tok.ptr, d_hist.ptr, d_pos.ptr, 16, None, H, d_x.ptr)):
         with pytest.raises(_lib.RbnError) as e:
             check(ctx.lib.rbn_greedy_next_f32(ctx.handle, *args))
         assert e.value.code == _lib.RBN_ERR_INVALID
+    with pytest.raises(_lib.RbnError):   # a history needs its capacity
+        check(ctx.lib.rbn_argmax_f32(ctx.handle, d_v.ptr, V, d_tok.ptr, d_hist.ptr, d_pos.ptr, 0))
+
+
+def device_flags(ctx):
+    f = C.c_uint32()
+    check(ctx.lib.rbn_device_flags(ctx.handle, C.byref(f)))
+    return f.value
+
+
+def test_history_capacity_is_respected(ctx):
+    # at the end of the history nothing is written past it, the position stays, and the
+    # context's flag word says so; the kernel itself runs and exits normally
+    V, H, cap = 500, 64, 8
+    table = synth_normal(41, 1.0, (V, H))
+    v = synth_normal(42, 1.0, (V,))
+    v[123] = v.max() + 1
+    d_table, d_v = ctx.to_device(table), ctx.to_device(v)
+    guard = np.full(32, -7, np.int32)
+    d_hist, d_tok, d_x = ctx.to_device(guard), ctx.alloc(4), ctx.alloc(4 * H)
+    d_pos = ctx.to_device(np.array([cap - 2], np.int32))
+    assert device_flags(ctx) == 0
+    call = lambda: check(ctx.lib.rbn_greedy_next_f32(ctx.handle, d_v.ptr, V, d_tok.ptr, d_hist.ptr, d_pos.ptr,
+                                                     cap, d_table.ptr, H, d_x.ptr))
+    call()                                       # slot cap - 1: the last one that exists
+    assert d_pos.download(np.int32, 1)[0] == cap - 1 and device_flags(ctx) == 0
+    for _ in range(3):                           # beyond: refused on the device
+        call()
+    hist = d_hist.download(np.int32, 32)
+    assert d_pos.download(np.int32, 1)[0] == cap - 1
+    assert hist[cap - 1] == 123 and (hist[cap:] == -7).all() and (hist[:cap - 1] == -7).all()
+    assert d_tok.download(np.int32, 1)[0] == 123
+    assert device_flags(ctx) == _lib.FLAG_HISTORY_OVERFLOW
+    assert device_flags(ctx) == 0                # reading clears it
+    # rbn_argmax_f32 with a position outside the history (also a negative one)
+    for bad in (cap, cap + 100, -1):
+        d_p = ctx.to_device(np.array([bad], np.int32))
+        check(ctx.lib.rbn_argmax_f32(ctx.handle, d_v.ptr, V, d_tok.ptr, d_hist.ptr, d_p.ptr, cap))
+        assert device_flags(ctx) == _lib.FLAG_HISTORY_OVERFLOW
+    assert (d_hist.download(np.int32, 32) == hist).all()
+
+
+def test_decoder_refuses_to_pass_max_seq(ctx):
+    # host-side checks: nothing is launched for a prompt or a decode that would leave the caches
+    cfg = DecoderConfig(layers=1, hidden=256, heads=2, head_dim=128, ffn=384, vocab=1000, max_seq=16)
+    dec = BitNetDecoder(ctx, cfg, max_batch_tokens=16)
+    dec.init_random(seed=3)
+    with pytest.raises(ValueError, match="max_seq"):
+        dec.prefill(np.arange(16, dtype=np.int32))
+    with pytest.raises(ValueError):
+        dec.prefill(np.zeros(0, dtype=np.int32))
+    dec.prefill(np.arange(12, dtype=np.int32))
+    with pytest.raises(ValueError, match="max_seq"):
+        dec.decode(4, use_graph=False)
+    toks, _ = dec.decode(3, use_graph=False)     # positions 13, 14, 15: the last that exist
+    assert len(toks) == 3 and device_flags(ctx) == 0
+    with pytest.raises(ValueError, match="max_seq"):
+        dec.decode(1, use_graph=False)
 
 
 @pytest.mark.parametrize("M,pos0,heads", [(1, 0, 2), (1, 130, 3), (6, 0, 2), (5, 250, 2), (1, 1023, 1),
@@ -265,3 +324,44 @@ def test_tiny_decoder_matches_numpy_model(ctx):
     dec.prefill(prompt)
     toks2, _ = dec.decode(6, use_graph=False)
     assert list(toks2) == list(toks)
+
+
+def test_full_size_decoder_graph_equals_eager(ctx):
+    """The 2B-class configuration at its real size (24 layers, hidden 2560, 20 heads of 128, FFN
+    6912, vocabulary 32000, 512-token prompt): no CPU model runs at this size, so what is
+    checked are the exact properties - the captured step replays to the same tokens as the
+    kernel-by-kernel step, two runs give identical tokens and logits, and the f16 K/V rows the
+    steps wrote are the same bits either way."""
+    cfg = DecoderConfig(max_seq=512 + 40)
+    dec = BitNetDecoder(ctx, cfg, max_batch_tokens=512)
+    dec.init_random(seed=4)
+    prompt = (np.arange(512, dtype=np.int64) * 7919 % cfg.vocab).astype(np.int32)
+    n_new = 24
+    row = cfg.head_dim
+    runs = []
+    for use_graph in (True, False, True):
+        print("full-size decoder, graph =", use_graph, flush=True)
+        dec.prefill(prompt)
+        first = dec.generated(1)[0]
+        logits0 = dec.last_logits()
+        toks, _ = dec.decode(n_new, use_graph=use_graph)
+        kv = []
+        for layer in (0, cfg.layers - 1):
+            for cache in (dec.kcache[layer], dec.vcache[layer]):
+                # head 0 and the last head, the rows of the prompt's tail and of the new tokens
+                for head in (0, cfg.heads - 1):
+                    off = 2 * (head * cfg.max_seq + 500) * row
+                    kv.append(cache.download(np.uint16, (12 + n_new) * row, offset_bytes=off))
+        runs.append((first, logits0, np.array(toks), dec.last_logits(), kv))
+    assert np.isfinite(runs[0][1]).all() and np.isfinite(runs[0][3]).all()
+    assert len(set(runs[0][2].tolist())) > 1, "a constant continuation would prove nothing"
+    for other in runs[1:]:
+        assert other[0] == runs[0][0]
+        assert (other[1].view(np.uint32) == runs[0][1].view(np.uint32)).all()
+        assert (other[2] == runs[0][2]).all(), (other[2], runs[0][2])
+        assert (other[3].view(np.uint32) == runs[0][3].view(np.uint32)).all()
+        for a, b in zip(other[4], runs[0][4]):
+            assert (a == b).all()
+    f = C.c_uint32()
+    check(ctx.lib.rbn_device_flags(ctx.handle, C.byref(f)))
+    assert f.value == 0

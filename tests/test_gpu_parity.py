@@ -136,6 +136,23 @@ def test_quantize_ternary_bit_exact(ctx, shape, sigma):
     assert (packed == t.packed_data).all()
 
 
+@pytest.mark.parametrize("shape,sigma", [((4096, 11008), 0.02), ((8192, 28672), 0.015)])
+def test_quantize_ternary_bit_exact_full_shapes(ctx, shape, sigma):
+    # the FFN up/gate matrix of the decode sweep and the 235 M-weight large-layer matrix: every
+    # packed byte, the threshold and the scale against the oracle's sequential sums (which
+    # drift to 0.83 and 0.34 of the true sum at these sizes, so a tree sum cannot pass)
+    say("quantize full shape", shape)
+    w = synth_normal(0x5EED1001 + shape[1], sigma, shape)
+    t = O.quantize_ternary(w)
+    true_thr = np.abs(w).astype(np.float64).mean() * 0.7
+    assert float(t.threshold) < (0.9 if shape[0] == 4096 else 0.4) * true_thr
+    _, packed, scale, thr, cnt = device_quantize(ctx, w)
+    assert bits(thr) == bits(t.threshold)
+    assert cnt == t.survivors
+    assert bits(scale) == bits(t.scale)
+    assert packed.size == w.size // 4 and (packed == t.packed_data).all()
+
+
 def test_quantize_tree_mode_is_close_but_flagged(ctx):
     w = synth_normal(3, 0.02, (1 << 22,))
     _, packed, scale, thr, cnt = device_quantize(ctx, w, TREE)
@@ -361,6 +378,74 @@ def test_gemm_mfma_more_than_one_round(ctx, M, K, N):
     w = synth_normal(0x5EED100A + N, 0.02, (K, N))
     res = run_matmul(ctx, ctx.gemm, x, w)
     check_against_oracle(x, w, *res, literal=False)
+
+
+def test_prefill_gemm_full_shape(ctx):
+    # the prefill configuration at its own shape: M=2048, K=4096, N=11008, through the MFMA
+    # kernel directly and through the dispatcher (which must pick it)
+    M, K, N = 2048, 4096, 11008
+    say("gemm full prefill shape", M, K, N)
+    assert ctx.lib.rbn_matmul_kernel_choice(M, K, N) == 2
+    x = synth_normal(0x5EED0004, 1.0, (M, K))
+    w = synth_normal(0x5EED1004, 0.02, (K, N))
+    res = run_matmul(ctx, ctx.gemm, x, w)
+    check_against_oracle(x, w, *res, literal=False)
+    again = run_matmul(ctx, ctx.matmul, x, w)
+    assert (again[1] == res[1]).all() and same_bits(again[0], res[0])
+
+
+class LargeLayer:
+    """K=8192, N=28672 weights (sigma 0.015), ternarised by the oracle and by the device once."""
+
+    def __init__(self, ctx):
+        self.K, self.N = 8192, 28672
+        say("large layer: generating and ternarising 8192 x 28672")
+        w = synth_normal(0x5EED1005, 0.015, (self.K, self.N))
+        self.t, self.vals = oracle_weights(w)
+        d_w = ctx.to_device(w)
+        d_p, self.w_scale, self.w_thr, self.survivors = ctx.quantize_ternary(d_w, w.size)
+        self.packed = d_p.download(np.uint8, w.size // 4)
+        self.d_tiled = ctx.tile_weights(d_p, self.K, self.N)
+        ctx.sync()
+        d_w.free()
+        d_p.free()
+        self.vals_f32 = self.vals.astype(np.float32)   # 128 * K < 2^24: f32 products are exact
+
+
+@pytest.fixture(scope="module")
+def large_layer(ctx):
+    ll = LargeLayer(ctx)
+    yield ll
+    ll.d_tiled.free()
+
+
+def test_large_layer_packed_bytes(ctx, large_layer):
+    ll = large_layer
+    assert bits(ll.w_thr) == bits(ll.t.threshold) and bits(ll.w_scale) == bits(ll.t.scale)
+    assert ll.survivors == ll.t.survivors
+    assert (ll.packed == ll.t.packed_data).all()
+    words = ll.d_tiled.download(np.uint32, ctx.lib.rbn_tiled_bytes(ll.K, ll.N) // 4)
+    assert (decode_tiled(words, ll.K, ll.N) == ll.vals).all()
+
+
+@pytest.mark.parametrize("M,entry,kernel", [(1, "gemv", 0), (1, "matmul", 0), (8, "matmul", 1), (64, "matmul", 2),
+                                            (64, "gemm", 2)])
+def test_large_layer_matmul(ctx, large_layer, M, entry, kernel):
+    # every token count of the large-layer configuration through the kernel the dispatcher
+    # picks for it (M=1: dot8 GEMV, M=8: streaming small-batch kernel, M=64: MFMA tiles)
+    ll = large_layer
+    say("large layer matmul", M, entry)
+    if entry == "matmul":
+        assert ctx.lib.rbn_matmul_kernel_choice(M, ll.K, ll.N) == kernel
+    x = synth_normal(0x5EED0005 + M, 1.0, (M, ll.K))
+    acts = ctx.act_quant_i8(ctx.to_device(x), M, ll.K)
+    d_out, d_acc = getattr(ctx, entry)(acts, ll.d_tiled, ll.w_scale, M, ll.K, ll.N, want_acc=True)
+    q, s, rs = O.act_quant_i8(x)
+    assert (acts[0].download(np.int8, M * ll.K).reshape(M, ll.K) == q).all()
+    want_acc = np.rint(q.astype(np.float32) @ ll.vals_f32).astype(np.int32)
+    want_out = epilogue(want_acc, s, ll.t.scale)
+    assert (d_acc.download(np.int32, M * ll.N).reshape(M, ll.N) == want_acc).all()
+    assert same_bits(d_out.download(np.float32, M * ll.N).reshape(M, ll.N), want_out)
 
 
 @pytest.mark.parametrize("M", [1, 2, 3, 7, 16, 17, 31, 32, 33, 48, 64])

@@ -221,6 +221,23 @@ int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_sc
 int rbn_gemm_t2_i8_mfma(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
                         const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
                         uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);
+/* rbn_gemm_t2_i8_skinny for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
+ * the reference.  Same arguments, same kernels, same bits; the difference is where narrow
+ * matrices exchange their split-k partial tiles: in a static device array of the library
+ * (RBN_STATIC_SCRATCH_BYTES per GPU, held until the process ends) instead of the workspace a
+ * context allocates.  Nothing on this path calls hipMalloc, hipFree or any allocating routine.
+ * A shape whose launch would need more than RBN_STATIC_SCRATCH_TILES partial tiles of 16 x 64
+ * int32 (ceil(N/64) * splits * ceil(M/16), only when the matrix is narrow enough to be split
+ * along k; M <= 16 always fits) is refused with RBN_ERR_UNSUPPORTED and a message that names
+ * the need and the limit.  All calls on one GPU share the array, from whichever context:
+ * calls that overlap on one GPU race and give wrong results; calls on one context are
+ * serialised by the context's lock and stream. */
+#define RBN_STATIC_SCRATCH_TILES 1024
+#define RBN_STATIC_SCRATCH_BYTES (RBN_STATIC_SCRATCH_TILES * 4096 + 128 * 4)
+int rbn_gemm_t2_i8_skinny_static(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
+                                 const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
+                                 uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);
 int rbn_matmul_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
                      const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
                      uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);

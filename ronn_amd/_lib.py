@@ -92,6 +92,7 @@ SIGNATURES = {
     "rbn_gemv_t2_i8_kernel_time": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp,
                                              C.POINTER(C.c_float)]),
     "rbn_gemm_t2_i8_skinny": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
+    "rbn_gemm_t2_i8_skinny_static": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
     "rbn_gemm_t2_i8_mfma": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
     "rbn_bitlinear_gemv_f32": (C.c_int, [_vp, _vp, _vp, _vp, C.c_float, _vp, C.c_float, _u64, _u64, _vp, _vp]),
     "rbn_embed_f32": (C.c_int, [_vp, _vp, _vp, _u64, _u64, _u64, _vp]),

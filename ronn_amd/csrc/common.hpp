@@ -43,8 +43,9 @@ constexpr int RBN_SPLITK_GROUPS = 1024;
 int rbn_fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
 void rbn_clear_error();
 
-// Raises the dynamic-LDS limit of the small-batch kernels (once per process and device).
-int rbn_skinny_prepare();
+// Per-device set-up of the small-batch kernels (dynamic-LDS limit, address of their static
+// scratch array); called with `device` current.
+int rbn_skinny_prepare(int device);
 
 // Ensures ctx->ws has at least `bytes` bytes; returns it through *out.
 int rbn_workspace(rbn_ctx *ctx, size_t bytes, void **out);

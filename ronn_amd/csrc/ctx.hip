@@ -101,7 +101,7 @@ int rbn_ctx_create(int device, rbn_ctx **out) {
         rbn_ctx_destroy(ctx);
         return rc;
     }
-    const int prep = rbn_skinny_prepare();
+    const int prep = rbn_skinny_prepare(device);
     if (prep != RBN_OK) {
         rbn_ctx_destroy(ctx);
         return prep;

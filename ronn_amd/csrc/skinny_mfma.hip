@@ -340,9 +340,26 @@ int launch_d(hipStream_t stream, const Args &a) {
 
 }  // namespace
 
-// Called once per context, outside any stream capture, for every instantiation that
-// launch_d can pick.
-int rbn_skinny_prepare() {
+// Scratch of the entry point that allocates nothing (rbn_gemm_t2_i8_skinny_static): partial
+// tiles first, then the ticket counters.  One copy per GPU, held until the process ends.
+constexpr int kStaticTiles = 1024;   // partial tiles of 16 x 64 int32 (4 KiB each): 4 MiB
+constexpr int kStaticGroups = 128;   // ticket counters (a split launch has fewer than 128 column groups)
+constexpr size_t kStaticBytes = (size_t)kStaticTiles * 4096 + (size_t)kStaticGroups * sizeof(unsigned);
+static __device__ __align__(256) unsigned char scratch[kStaticBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_lock;
+static void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, 0 until prepared
+
+__global__ void clear_tickets_kernel(unsigned *tickets, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) tickets[i] = 0u;
+}
+
+// Called once per context, with the context's device current and outside any stream capture:
+// raises the dynamic-LDS limit of every instantiation that launch_d can pick and looks up this
+// device's copy of the static scratch array.
+int rbn_skinny_prepare(int device) {
     const hipError_t results[] = {
         allow_large_lds<1, 1, 2, false>(), allow_large_lds<1, 1, 4, false>(),
         allow_large_lds<1, 1, 8, false>(), allow_large_lds<1, 1, 8, true>(),
@@ -355,19 +372,32 @@ int rbn_skinny_prepare() {
         if (e != hipSuccess)
             return rbn_fail(RBN_ERR_HIP, "hipFuncSetAttribute(max dynamic LDS) failed: %s",
                             hipGetErrorString(e));
+    if (device < 0 || device >= kMaxDevices)
+        return rbn_fail(RBN_ERR_UNSUPPORTED, "device index %d beyond the %d this library keeps scratch for",
+                        device, kMaxDevices);
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (g_scratch_ptr[device] == nullptr) {
+        void *ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr)
+            return rbn_fail(RBN_ERR_HIP, "hipGetSymbolAddress(scratch) failed on device %d: %s", device,
+                            hipGetErrorString(e));
+        g_scratch_ptr[device] = ptr;
+    }
     return RBN_OK;
 }
 
-extern "C" int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
-                                     const int32_t *d_rowsum, const uint32_t *d_tiled,
-                                     float w_scale, uint64_t M, uint64_t K, uint64_t N,
-                                     int32_t *d_acc, float *d_out) {
-    RBN_ENTER(ctx);
+// partials / tickets: the split-k exchange area and what it holds (tiles of 4 KiB, counters).
+// With `strict` a launch shape that does not fit is an error; otherwise the split is reduced
+// until it fits (any split gives the same bits).
+static int skinny_impl(rbn_ctx *ctx, const char *name, const int8_t *d_q, const float *d_act_scale,
+                       const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale, uint64_t M,
+                       uint64_t K, uint64_t N, int32_t *d_acc, float *d_out, void *partials,
+                       unsigned *tickets, int max_tiles, int max_groups, bool strict) {
     RBN_REQUIRE(M > 0 && K > 0 && N > 0, "M, K and N must be positive");
-    RBN_REQUIRE(M <= RBN_SKINNY_MAX_M, "rbn_gemm_t2_i8_skinny takes M <= %d (got %llu)",
-                RBN_SKINNY_MAX_M, (unsigned long long)M);
-    RBN_REQUIRE(d_q && d_act_scale && d_rowsum && d_tiled && d_out,
-                "null pointer in rbn_gemm_t2_i8_skinny");
+    RBN_REQUIRE(M <= RBN_SKINNY_MAX_M, "%s takes M <= %d (got %llu)", name, RBN_SKINNY_MAX_M,
+                (unsigned long long)M);
+    RBN_REQUIRE(d_q && d_act_scale && d_rowsum && d_tiled && d_out, "null pointer in %s", name);
     RBN_REQUIRE((((uintptr_t)d_q | (uintptr_t)d_tiled) & 15u) == 0,
                 "d_q and d_tiled must be 16-byte aligned");
     RBN_REQUIRE((((uintptr_t)d_out | (uintptr_t)d_acc) & 15u) == 0,
@@ -382,8 +412,8 @@ extern "C" int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const floa
     a.M = (int)M;
     a.Kpad = (int)rbn_kpad(K);
     a.N = (int)N;
-    a.partials = (int4 *)ctx->splitk_partials;
-    a.tickets = ctx->splitk_tickets;
+    a.partials = (int4 *)partials;
+    a.tickets = tickets;
     a.acc = d_acc;
     a.out = d_out;
     const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
@@ -413,10 +443,19 @@ extern "C" int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const floa
         const int want = (steps + per - 1) / per;
         if (want < splits) splits = want;
     }
-    // the workspace holds RBN_SPLITK_TILES tiles of 16 x 64 int32 and one ticket per group
-    while (splits > 1 &&
-           ((int64_t)a.groups * splits * mt * ng > RBN_SPLITK_TILES || a.groups > RBN_SPLITK_GROUPS))
-        --splits;
+    // the exchange area holds max_tiles tiles of 16 x 64 int32 and one ticket per group
+    if (strict) {
+        if (splits > 1 && ((int64_t)a.groups * splits * mt * ng > max_tiles || a.groups > max_groups))
+            return rbn_fail(RBN_ERR_UNSUPPORTED,
+                            "%s: M=%llu K=%llu N=%llu needs %lld partial tiles and %d counters; the static "
+                            "scratch holds %d tiles (%zu bytes) and %d counters - use rbn_gemm_t2_i8_skinny",
+                            name, (unsigned long long)M, (unsigned long long)K, (unsigned long long)N,
+                            (long long)a.groups * splits * mt * ng, a.groups, max_tiles,
+                            (size_t)max_tiles * 4096, max_groups);
+    } else {
+        while (splits > 1 && ((int64_t)a.groups * splits * mt * ng > max_tiles || a.groups > max_groups))
+            --splits;
+    }
     const int steps_per_split = (steps + splits - 1) / splits;
     int waves = (steps_per_split + 3) / 4;
     if (waves > max_w) waves = max_w;
@@ -424,6 +463,10 @@ extern "C" int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const floa
     if (waves < 1) waves = 1;
     a.splits = splits;
     a.waves = waves;
+    if (strict && splits > 1) {
+        // the array keeps the last call's contents: the counters this launch draws from start at zero
+        clear_tickets_kernel<<<dim3(1), dim3(kStaticGroups), 0, ctx->stream>>>(tickets, kStaticGroups);
+    }
     int rc;
     switch (mt) {
         case 1: rc = launch_d<1, 1>(ctx->stream, a); break;
@@ -433,4 +476,34 @@ extern "C" int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const floa
     RBN_CHECK(rc);
     RBN_HIP(hipGetLastError());
     return RBN_OK;
+}
+
+extern "C" int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
+                                     const int32_t *d_rowsum, const uint32_t *d_tiled,
+                                     float w_scale, uint64_t M, uint64_t K, uint64_t N,
+                                     int32_t *d_acc, float *d_out) {
+    RBN_ENTER(ctx);
+    return skinny_impl(ctx, "rbn_gemm_t2_i8_skinny", d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N,
+                       d_acc, d_out, ctx->splitk_partials, ctx->splitk_tickets, RBN_SPLITK_TILES,
+                       RBN_SPLITK_GROUPS, false);
+}
+
+// The same kernels with the split-k exchange area in this file's static device array instead of
+// memory the context allocated: no allocation anywhere on this path.
+extern "C" int rbn_gemm_t2_i8_skinny_static(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
+                                            const int32_t *d_rowsum, const uint32_t *d_tiled,
+                                            float w_scale, uint64_t M, uint64_t K, uint64_t N,
+                                            int32_t *d_acc, float *d_out) {
+    RBN_ENTER(ctx);
+    void *base = nullptr;
+    if (ctx->device >= 0 && ctx->device < kMaxDevices) {
+        std::lock_guard<std::mutex> hold(g_scratch_lock);
+        base = g_scratch_ptr[ctx->device];
+    }
+    if (base == nullptr)
+        return rbn_fail(RBN_ERR_HIP, "the static scratch of device %d was never looked up", ctx->device);
+    unsigned *tickets = reinterpret_cast<unsigned *>(static_cast<unsigned char *>(base) +
+                                                     (size_t)kStaticTiles * 4096);
+    return skinny_impl(ctx, "rbn_gemm_t2_i8_skinny_static", d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M,
+                       K, N, d_acc, d_out, base, tickets, kStaticTiles, kStaticGroups, true);
 }

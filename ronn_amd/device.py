@@ -219,6 +219,11 @@ class Context:
         return self._mm(self.lib.rbn_gemm_t2_i8_skinny, acts, d_tiled, w_scale, M, K, N, want_acc,
                         d_out, d_acc)
 
+    def skinny_static(self, acts, d_tiled, w_scale, M, K, N, want_acc=False, d_out=None, d_acc=None):
+        """rbn_gemm_t2_i8_skinny with the split-k exchange in the library's static device array."""
+        return self._mm(self.lib.rbn_gemm_t2_i8_skinny_static, acts, d_tiled, w_scale, M, K, N, want_acc,
+                        d_out, d_acc)
+
     def gemm(self, acts, d_tiled, w_scale, M, K, N, want_acc=False, d_out=None, d_acc=None):
         return self._mm(self.lib.rbn_gemm_t2_i8_mfma, acts, d_tiled, w_scale, M, K, N, want_acc,
                         d_out, d_acc)

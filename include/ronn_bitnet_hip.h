@@ -215,6 +215,29 @@ int rbn_gemv_t2_i8_kernel_time(rbn_ctx *ctx, const int8_t *d_q, const float *d_a
                                const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
                                uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out,
                                float *h_kernel_us);
+/* Several independent decode GEMVs of one shape in ONE launch (q/k/v or gate/up projections of
+ * a token, the experts or adapters of a layer, the same layer of several sequences).  Every
+ * problem is a complete rbn_gemv_t2_i8 with its own activations, weights and outputs, and
+ * gives the bits rbn_gemv_t2_i8 gives.  What the grouping buys is time: a single GEMV of a few
+ * MB is shorter than the gap between two launches plus the ramp of its first loads, and in one
+ * grid the problems overlap.  h_problems is a HOST array of `count` descriptors (1 to
+ * RBN_GEMV_GROUP_MAX); the pointers inside are device pointers.  The descriptors are copied
+ * into the launch's arguments, so the array may be reused as soon as the call returns and the
+ * call can be captured in a graph.  No reference counterpart (the reference multiplies one
+ * pair of tensors per execute(), kernels.rs:271-283). */
+#define RBN_GEMV_GROUP_MAX 32
+typedef struct rbn_gemv_problem {
+    const int8_t *d_q;        /* [M, rbn_act_pitch(K)] int8 */
+    const float *d_act_scale; /* [M] */
+    const int32_t *d_rowsum;  /* [M] */
+    const uint32_t *d_tiled;  /* tiled weights [K,N] */
+    float *d_out;             /* [M,N] f32 */
+    int32_t *d_acc;           /* [M,N] int32 accumulators, or NULL */
+    float w_scale;
+    uint32_t reserved;        /* set to 0 */
+} rbn_gemv_problem;
+int rbn_gemv_t2_i8_grouped(rbn_ctx *ctx, const rbn_gemv_problem *h_problems, uint64_t count,
+                           uint64_t M, uint64_t K, uint64_t N);
 int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
                           const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
                           uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);
@@ -334,6 +357,13 @@ enum rbn_probe_operands {
     RBN_PROBE_I8_I8 = 2       /* random int8 x random int8 */
 };
 int rbn_probe_mfma_i8(rbn_ctx *ctx, int operand_kind, double *h_tops);
+/* The floor of a streaming kernel on this machine, for pricing the GEMV: one launch that does
+ * nothing (rbn_probe_empty_launch), and one that only reads `bytes` of d_src with the GEMV's
+ * access pattern (16-byte loads, 4 KiB of consecutive memory per wave; non-temporal or
+ * plain) and stores nothing.  Asynchronous on the context's stream and capturable, so they
+ * are timed the way the GEMV is (graph replay, rbn_timer_*). */
+int rbn_probe_empty_launch(rbn_ctx *ctx);
+int rbn_probe_stream_read(rbn_ctx *ctx, const void *d_src, uint64_t bytes, int nontemporal);
 
 /* ---- synthetic inputs (host) ----------------------------------------------- */
 /* out[i] = (float)(sigma * z_i), z_i standard normal from a counter-based

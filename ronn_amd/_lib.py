@@ -22,6 +22,7 @@ RBN_ERR_NO_DEVICE = -5
 SUM_STRICT_SEQ = 0
 SUM_TREE = 1
 GEMV_MAX_M = 16
+GEMV_GROUP_MAX = 32
 FLAG_HISTORY_OVERFLOW = 1
 
 # dtype codes of rbn_tensor_bytes (declaration order of the reference's DataType)
@@ -38,6 +39,20 @@ class DeviceInfo(C.Structure):
         ("mem_bus_bits", C.c_int),
         ("hbm_bytes", C.c_uint64),
         ("l2_bytes", C.c_uint64),
+    ]
+
+
+class GemvProblem(C.Structure):
+    """rbn_gemv_problem: one GEMV of a grouped launch (device pointers)."""
+    _fields_ = [
+        ("d_q", C.c_void_p),
+        ("d_act_scale", C.c_void_p),
+        ("d_rowsum", C.c_void_p),
+        ("d_tiled", C.c_void_p),
+        ("d_out", C.c_void_p),
+        ("d_acc", C.c_void_p),
+        ("w_scale", C.c_float),
+        ("reserved", C.c_uint32),
     ]
 
 
@@ -91,6 +106,7 @@ SIGNATURES = {
     "rbn_gemv_t2_i8": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
     "rbn_gemv_t2_i8_kernel_time": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp,
                                              C.POINTER(C.c_float)]),
+    "rbn_gemv_t2_i8_grouped": (C.c_int, [_vp, C.POINTER(GemvProblem), _u64, _u64, _u64, _u64]),
     "rbn_gemm_t2_i8_skinny": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
     "rbn_gemm_t2_i8_skinny_static": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
     "rbn_gemm_t2_i8_mfma": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
@@ -107,6 +123,8 @@ SIGNATURES = {
     "rbn_add_i32": (C.c_int, [_vp, _vp, C.c_int32]),
     "rbn_synth_normal_device_f32": (C.c_int, [_vp, _u64, C.c_float, _vp, _u64]),
     "rbn_probe_mfma_i8": (C.c_int, [_vp, C.c_int, C.POINTER(C.c_double)]),
+    "rbn_probe_empty_launch": (C.c_int, [_vp]),
+    "rbn_probe_stream_read": (C.c_int, [_vp, _vp, _u64, C.c_int]),
     "rbn_matmul_kernel_choice": (C.c_int, [_u64, _u64, _u64]),
     "rbn_matmul_t2_i8": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
     "rbn_execute_ternary_matmul": (C.c_int, [_vp, _vp, _vp, _u64, _u64, _u64, C.c_int, _vp, _vp]),

@@ -301,6 +301,10 @@ int rbn_graph_end_capture(rbn_ctx *ctx, rbn_graph **out) {
         (void)hipGraphDestroy(g);
         return rbn_fail(RBN_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
     }
+    // Resources of the executable graph go to the device now, not inside its first launch
+    // (a launch-bound sequence would otherwise see one slow first replay).  Best effort.
+    (void)hipGraphUpload(exec, ctx->stream);
+    (void)hipGetLastError();
     rbn_graph *r = new (std::nothrow) rbn_graph();
     if (!r) {
         (void)hipGraphExecDestroy(exec);

@@ -74,15 +74,16 @@ __device__ __forceinline__ uint4 ld_w(const uint4 *p) {
 // MT tokens, KS waves per column quad, L weight loads in flight per lane and round.
 // EXACT: the k-blocks fit one pass and are a multiple of 64 * L, so no index of the
 // loop needs a clamp and no block a mask.
+// `block` is the workgroup's index inside its problem (blockIdx.x for a single GEMV).
 template <int MT, int KS, int L, bool EXACT>
-__global__ __launch_bounds__(kThreads) void gemv_t2_i8_kernel(
+__device__ __forceinline__ void gemv_body(
     const uint4 *__restrict__ q4,         // [M][KB]: 16 int8 each
     const float *__restrict__ act_scale,  // [M]
     const int32_t *__restrict__ rowsum,   // [M]
     const uint4 *__restrict__ w4,         // [nquads][KB]
     float w_scale, int M, int KB, int KC /* k-blocks staged per pass */, int N, int nquads,
     int vec_store /* N % 4 == 0 and the outputs are 16-byte aligned */,
-    int32_t *__restrict__ acc_out, float *__restrict__ out) {
+    int32_t *__restrict__ acc_out, float *__restrict__ out, const int block) {
     constexpr int QPB = kWaves / KS;  // quads per workgroup
     extern __shared__ uint4 s_a[];  // MT * KC staged activation blocks (4-bit planes)
     __shared__ int s_part[KS > 1 ? kWaves * MT * 4 : 1];
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(kThreads) void gemv_t2_i8_kernel(
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int quad_local = wave / KS, slice = wave % KS;
-    int quad = blockIdx.x * QPB + quad_local;
+    int quad = block * QPB + quad_local;
     const bool active = quad < nquads;
     quad = active ? quad : nquads - 1;
     const uint4 *wq = w4 + (size_t)quad * KB;
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(kThreads) void gemv_t2_i8_kernel(
         __syncthreads();
         for (int idx = tid; idx < QPB * MT * 4; idx += kThreads) {
             const int ql = idx / (MT * 4), m = (idx / 4) % MT, c = idx % 4;
-            const int qd = blockIdx.x * QPB + ql;
+            const int qd = block * QPB + ql;
             const int n = qd * 4 + c;
             if (qd < nquads && m < M && n < N) {
                 int total = 0;
@@ -271,7 +272,37 @@ __global__ __launch_bounds__(kThreads) void gemv_t2_i8_kernel(
     }
 }
 
+template <int MT, int KS, int L, bool EXACT>
+__global__ __launch_bounds__(kThreads) void gemv_t2_i8_kernel(
+    const uint4 *__restrict__ q4, const float *__restrict__ act_scale, const int32_t *__restrict__ rowsum,
+    const uint4 *__restrict__ w4, float w_scale, int M, int KB, int KC, int N, int nquads, int vec_store,
+    int32_t *__restrict__ acc_out, float *__restrict__ out) {
+    gemv_body<MT, KS, L, EXACT>(q4, act_scale, rowsum, w4, w_scale, M, KB, KC, N, nquads, vec_store, acc_out,
+                                out, (int)blockIdx.x);
+}
+
+// Several independent GEMVs of one shape in one launch: workgroup b works on problem
+// b / blocks_per_problem.  The problems' pointers travel in the kernel arguments (a workgroup
+// reads its own with scalar loads), so nothing has to be uploaded before the launch.  Back to
+// back in one grid the problems overlap: the next one's first loads are in flight while the
+// previous one's last waves reduce and store, which a launch of its own cannot do.
+struct GroupArgs {
+    rbn_gemv_problem p[RBN_GEMV_GROUP_MAX];
+};
+
+template <int MT, int KS, int L, bool EXACT>
+__global__ __launch_bounds__(kThreads) void gemv_t2_i8_grouped_kernel(
+    const GroupArgs g, int blocks_per_problem, int M, int KB, int KC, int N, int nquads, int vec_store) {
+    const int p = __builtin_amdgcn_readfirstlane((int)blockIdx.x / blocks_per_problem);
+    const int block = (int)blockIdx.x - p * blocks_per_problem;
+    const rbn_gemv_problem &d = g.p[p];
+    gemv_body<MT, KS, L, EXACT>((const uint4 *)d.d_q, d.d_act_scale, d.d_rowsum, (const uint4 *)d.d_tiled,
+                                d.w_scale, M, KB, KC, N, nquads, vec_store, d.d_acc, d.d_out, block);
+}
+
 struct Args {
+    const GroupArgs *group = nullptr;  // set: a grouped launch of `count` problems
+    int count = 1;
     const uint4 *q4;
     const float *act_scale;
     const int32_t *rowsum;
@@ -286,8 +317,23 @@ struct Args {
 template <int MT, int KS, int L>
 void launch(hipStream_t stream, const Args &a) {
     constexpr int QPB = kWaves / KS;
-    dim3 grid((unsigned)((a.nquads + QPB - 1) / QPB));
+    const int blocks = (a.nquads + QPB - 1) / QPB;
+    dim3 grid((unsigned)blocks);
     const size_t lds = (size_t)MT * a.KC * 16;
+    const bool exact = KS == 1 && MT <= 4 && a.KC == a.KB && a.KB % (64 * L) == 0;
+    if (a.group) {
+        dim3 ggrid((unsigned)(blocks * a.count));
+        if constexpr (KS == 1 && MT <= 4) {
+            if (exact) {
+                gemv_t2_i8_grouped_kernel<MT, KS, L, true><<<ggrid, dim3(kThreads), lds, stream>>>(
+                    *a.group, blocks, a.M, a.KB, a.KC, a.N, a.nquads, a.vec_store);
+                return;
+            }
+        }
+        gemv_t2_i8_grouped_kernel<MT, KS, L, false><<<ggrid, dim3(kThreads), lds, stream>>>(
+            *a.group, blocks, a.M, a.KB, a.KC, a.N, a.nquads, a.vec_store);
+        return;
+    }
     // with events given the launch records the kernel's own begin and end timestamps in them
     auto go = [&](auto kernel) {
         if (a.ev_begin)
@@ -299,7 +345,7 @@ void launch(hipStream_t stream, const Args &a) {
                                                          a.KB, a.KC, a.N, a.nquads, a.vec_store, a.acc, a.out);
     };
     if constexpr (KS == 1 && MT <= 4) {
-        if (a.KC == a.KB && a.KB % (64 * L) == 0) {
+        if (exact) {
             go(gemv_t2_i8_kernel<MT, KS, L, true>);
             return;
         }
@@ -340,6 +386,8 @@ void launch_ks(hipStream_t stream, const Args &a, int ks) {
 
 }  // namespace
 
+static void shape_and_launch(hipStream_t stream, Args &a);
+
 static int gemv_impl(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale, const int32_t *d_rowsum,
                      const uint32_t *d_tiled, float w_scale, uint64_t M, uint64_t K, uint64_t N,
                      int32_t *d_acc, float *d_out, float *h_kernel_us) {
@@ -368,6 +416,20 @@ static int gemv_impl(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale, 
         a.ev_end = ctx->ev_stop;
     }
     a.vec_store = N % 4 == 0 && (((uintptr_t)d_out | (uintptr_t)d_acc) & 15u) == 0;
+    shape_and_launch(ctx->stream, a);
+    RBN_HIP(hipGetLastError());
+    if (h_kernel_us) {
+        float ms = 0.0f;
+        RBN_HIP(hipEventSynchronize(ctx->ev_stop));
+        RBN_HIP(hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop));
+        *h_kernel_us = ms * 1000.0f;
+    }
+    return RBN_OK;
+}
+
+// Picks the launch shape for a.M, a.KB, a.nquads (a.KC is set here) and launches.
+static void shape_and_launch(hipStream_t stream, Args &a) {
+    const int M = a.M;
     const int mt = M == 1 ? 1 : M == 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16;
     // k-blocks whose staged activations fit the LDS budget in one pass
     const int kc_cap = kLdsBudget / 16 / mt;
@@ -388,20 +450,12 @@ static int gemv_impl(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale, 
             ks *= 2;
     }
     switch (mt) {
-        case 1: launch_ks<1>(ctx->stream, a, ks); break;
-        case 2: launch_ks<2>(ctx->stream, a, ks); break;
-        case 4: launch_ks<4>(ctx->stream, a, ks); break;
-        case 8: launch_ks<8>(ctx->stream, a, ks); break;
-        default: launch_ks<16>(ctx->stream, a, ks); break;
+        case 1: launch_ks<1>(stream, a, ks); break;
+        case 2: launch_ks<2>(stream, a, ks); break;
+        case 4: launch_ks<4>(stream, a, ks); break;
+        case 8: launch_ks<8>(stream, a, ks); break;
+        default: launch_ks<16>(stream, a, ks); break;
     }
-    RBN_HIP(hipGetLastError());
-    if (h_kernel_us) {
-        float ms = 0.0f;
-        RBN_HIP(hipEventSynchronize(ctx->ev_stop));
-        RBN_HIP(hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop));
-        *h_kernel_us = ms * 1000.0f;
-    }
-    return RBN_OK;
 }
 
 extern "C" int rbn_gemv_t2_i8(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
@@ -419,4 +473,47 @@ extern "C" int rbn_gemv_t2_i8_kernel_time(rbn_ctx *ctx, const int8_t *d_q, const
         return rbn_fail(RBN_ERR_INVALID, "h_kernel_us is NULL");
     }
     return gemv_impl(ctx, d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M, K, N, d_acc, d_out, h_kernel_us);
+}
+
+extern "C" int rbn_gemv_t2_i8_grouped(rbn_ctx *ctx, const rbn_gemv_problem *h_problems, uint64_t count,
+                                      uint64_t M, uint64_t K, uint64_t N) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(h_problems != nullptr, "h_problems is NULL");
+    RBN_REQUIRE(count >= 1 && count <= RBN_GEMV_GROUP_MAX, "rbn_gemv_t2_i8_grouped takes 1 to %d problems (got %llu)",
+                RBN_GEMV_GROUP_MAX, (unsigned long long)count);
+    RBN_REQUIRE(M > 0 && K > 0 && N > 0, "M, K and N must be positive");
+    RBN_REQUIRE(M <= RBN_GEMV_MAX_M, "rbn_gemv_t2_i8_grouped takes M <= %d (got %llu)", RBN_GEMV_MAX_M,
+                (unsigned long long)M);
+    RBN_REQUIRE(K <= (1ull << 30) && N <= (1ull << 30), "dimension too large");
+    GroupArgs g;
+    bool vec = N % 4 == 0;
+    for (uint64_t i = 0; i < count; ++i) {
+        const rbn_gemv_problem &p = h_problems[i];
+        RBN_REQUIRE(p.d_q && p.d_act_scale && p.d_rowsum && p.d_tiled && p.d_out,
+                    "null pointer in problem %llu of rbn_gemv_t2_i8_grouped", (unsigned long long)i);
+        RBN_REQUIRE((((uintptr_t)p.d_q | (uintptr_t)p.d_tiled) & 15u) == 0,
+                    "d_q and d_tiled of problem %llu must be 16-byte aligned", (unsigned long long)i);
+        vec = vec && (((uintptr_t)p.d_out | (uintptr_t)p.d_acc) & 15u) == 0;
+        g.p[i] = p;
+    }
+    for (uint64_t i = count; i < RBN_GEMV_GROUP_MAX; ++i) g.p[i] = h_problems[count - 1];
+    Args a;
+    a.group = &g;
+    a.count = (int)count;
+    a.q4 = nullptr;
+    a.act_scale = nullptr;
+    a.rowsum = nullptr;
+    a.w4 = nullptr;
+    a.w_scale = 0.0f;
+    a.M = (int)M;
+    a.KB = (int)(rbn_kpad(K) / 16);
+    a.N = (int)N;
+    a.nquads = (int)(rbn_npad(N) / 4);
+    a.acc = nullptr;
+    a.out = nullptr;
+    a.vec_store = vec;
+    RBN_REQUIRE((uint64_t)a.nquads * count < (1ull << 31), "too many workgroups");
+    shape_and_launch(ctx->stream, a);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
 }

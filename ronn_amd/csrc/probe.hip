@@ -39,7 +39,59 @@ __global__ __launch_bounds__(256, 2) void mfma_i8_probe_kernel(const v4i *__rest
     if (s == 0x7fffffff) sink[0] = s;  // keeps the loop alive; practically never true
 }
 
+// What a launch that only READS costs: workgroups of four waves, a lane loads four 16-byte
+// units 1 KiB apart (a wave reads 4 KiB of consecutive memory, a workgroup 16 KiB: the
+// GEMV's access pattern without its arithmetic, staging, reduction and stores).
+template <bool NT>
+__global__ __launch_bounds__(256) void stream_read_kernel(const uint4 *__restrict__ src, uint64_t units,
+                                                          uint32_t *__restrict__ sink) {
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    const uint64_t base = ((uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 256 + (threadIdx.x & 63);
+    uint4 v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint64_t at = base + 64 * i;
+        const uint4 *p = src + (at < units ? at : units - 1);
+        if (NT) {
+            const v4u t = __builtin_nontemporal_load(reinterpret_cast<const v4u *>(p));
+            v[i] = make_uint4(t.x, t.y, t.z, t.w);
+        } else {
+            v[i] = *p;
+        }
+    }
+    uint32_t x = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) x |= v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+    if (x == 0x9E3779B9u) sink[0] = x;  // keeps the loads alive; practically never true
+}
+
+__global__ void empty_kernel() {}
+
 }  // namespace
+
+extern "C" int rbn_probe_empty_launch(rbn_ctx *ctx) {
+    RBN_ENTER(ctx);
+    empty_kernel<<<dim3(1), dim3(64), 0, ctx->stream>>>();
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
+
+extern "C" int rbn_probe_stream_read(rbn_ctx *ctx, const void *d_src, uint64_t bytes, int nontemporal) {
+    RBN_ENTER(ctx);
+    RBN_REQUIRE(d_src != nullptr && bytes >= 16 && ((uintptr_t)d_src & 15u) == 0,
+                "rbn_probe_stream_read needs a 16-byte aligned buffer of at least 16 bytes");
+    const uint64_t units = bytes / 16, blocks = (units + 1023) / 1024;
+    RBN_REQUIRE(blocks < (1ull << 31), "buffer too large");
+    uint32_t *ws = ctx->dev_flags + 16;  // a word nobody reads (never written in practice)
+    if (nontemporal)
+        stream_read_kernel<true><<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>((const uint4 *)d_src, units,
+                                                                                      ws);
+    else
+        stream_read_kernel<false><<<dim3((unsigned)blocks), dim3(256), 0, ctx->stream>>>((const uint4 *)d_src, units,
+                                                                                       ws);
+    RBN_HIP(hipGetLastError());
+    return RBN_OK;
+}
 
 extern "C" int rbn_probe_mfma_i8(rbn_ctx *ctx, int operand_kind, double *h_tops) {
     RBN_ENTER(ctx);

@@ -190,6 +190,10 @@ class BitNetDecoder:
         check(lib.rbn_greedy_next_f32(hnd, self.logits.ptr, cfg.vocab, self.tokens.ptr, self.history.ptr,
                                       self.pos.ptr, cfg.max_seq, self.embed.ptr, cfg.hidden, self.x.ptr))
 
+    def launches_per_token(self) -> int:
+        """Kernel launches of one decode step (forward_one)."""
+        return 5 * self.cfg.layers + 2
+
     def forward(self, M: int):
         """Tokens self.tokens[0:M] at positions *pos .. *pos+M-1; leaves the logits of the
         last token in self.logits and its arg-max in self.tokens[0] and the history."""

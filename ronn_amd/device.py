@@ -215,6 +215,23 @@ class Context:
                                                   float(w_scale), M, K, N, None, d_out.ptr, C.byref(us)))
         return us.value
 
+    def gemv_problems(self, problems):
+        """Host array of rbn_gemv_problem from (acts, d_tiled, w_scale, d_out, d_acc or None) tuples."""
+        arr = (_lib.GemvProblem * len(problems))()
+        for p, (acts, d_tiled, w_scale, d_out, d_acc) in zip(arr, problems):
+            p.d_q, p.d_act_scale, p.d_rowsum = acts[0].ptr, acts[1].ptr, acts[2].ptr
+            p.d_tiled, p.d_out = d_tiled.ptr, d_out.ptr
+            p.d_acc = d_acc.ptr if d_acc is not None else None
+            p.w_scale, p.reserved = float(w_scale), 0
+        return arr
+
+    def gemv_grouped(self, problems, M, K, N, first=0, count=None):
+        """One launch of problems[first:first+count] (an array from gemv_problems), all of shape (M, K, N)."""
+        count = len(problems) - first if count is None else count
+        check(self.lib.rbn_gemv_t2_i8_grouped(
+            self.handle, C.cast(C.byref(problems, first * C.sizeof(_lib.GemvProblem)), C.POINTER(_lib.GemvProblem)),
+            count, M, K, N))
+
     def skinny(self, acts, d_tiled, w_scale, M, K, N, want_acc=False, d_out=None, d_acc=None):
         return self._mm(self.lib.rbn_gemm_t2_i8_skinny, acts, d_tiled, w_scale, M, K, N, want_acc,
                         d_out, d_acc)

@@ -318,6 +318,54 @@ def test_gemv_long_rows(ctx, M, K, N):
     check_against_oracle(x, w, *res, literal=False)
 
 
+@pytest.mark.parametrize("M,K,N,count", [(1, 4096, 1024, 32), (1, 2048, 2048, 5), (2, 1000, 77, 3), (4, 256, 520, 32),
+                                         (1, 11008, 256, 7), (16, 384, 130, 2), (1, 8192, 512, 1), (3, 640, 4096, 9)])
+def test_gemv_grouped_every_problem_is_its_own_gemv(ctx, M, K, N, count):
+    # `count` independent problems in one launch, each with its own activations, weights, scale
+    # and outputs: every one against the oracle's integers (through BLAS) and bit for bit against
+    # a launch of its own
+    say("gemv grouped", M, K, N, count)
+    problems, wants, singles = [], [], []
+    for j in range(count):
+        x = synth_normal(0x5EED0071 + 7 * j + M, 1.0 + 0.25 * j, (M, K))
+        w = synth_normal(0x5EED1071 + 5 * j + N, 0.02, (K, N))
+        d_p, w_scale, _, _ = ctx.quantize_ternary(ctx.to_device(w), w.size)
+        d_t = ctx.tile_weights(d_p, K, N)
+        acts = ctx.act_quant_i8(ctx.to_device(x), M, K)
+        t, vals = oracle_weights(w)
+        q, s, _ = O.act_quant_i8(x)
+        acc = exact_int_matmul(q, vals)
+        wants.append((acc, epilogue(acc, s, t.scale)))
+        assert bits(w_scale) == bits(t.scale)
+        d_out, d_acc = ctx.alloc(4 * M * N), (ctx.alloc(4 * M * N) if j % 2 == 0 else None)
+        ctx.lib.rbn_fill_u8(ctx.handle, d_out.ptr, 0xFF, 4 * M * N)
+        problems.append((acts, d_t, w_scale, d_out, d_acc))
+        singles.append(ctx.gemv(acts, d_t, w_scale, M, K, N)[0].download(np.float32, M * N))
+    ctx.gemv_grouped(ctx.gemv_problems(problems), M, K, N)
+    ctx.sync()
+    for j, ((acts, d_t, w_scale, d_out, d_acc), (want_acc, want_out)) in enumerate(zip(problems, wants)):
+        got = d_out.download(np.float32, M * N).reshape(M, N)
+        assert same_bits(got, want_out), j
+        assert same_bits(got.ravel(), singles[j]), j
+        if d_acc is not None:
+            assert (d_acc.download(np.int32, M * N).reshape(M, N) == want_acc).all(), j
+
+
+def test_gemv_grouped_refused_arguments(ctx):
+    d = ctx.alloc(4096)
+    probs = ctx.gemv_problems([((d, d, d), d, 1.0, d, None)] * 33)
+    for count, M in ((0, 1), (33, 1), (1, 0), (1, 17)):
+        rc = ctx.lib.rbn_gemv_t2_i8_grouped(ctx.handle, probs, count, M, 64, 64)
+        assert rc == _lib.RBN_ERR_INVALID, (count, M)
+    assert ctx.lib.rbn_gemv_t2_i8_grouped(ctx.handle, None, 1, 1, 64, 64) == _lib.RBN_ERR_INVALID
+    probs[1].d_out = None
+    assert ctx.lib.rbn_gemv_t2_i8_grouped(ctx.handle, probs, 2, 1, 64, 64) == _lib.RBN_ERR_INVALID
+    assert b"problem 1" in ctx.lib.rbn_last_error()
+    probs[1].d_out = d.ptr
+    probs[1].d_q = d.ptr + 4
+    assert ctx.lib.rbn_gemv_t2_i8_grouped(ctx.handle, probs, 2, 1, 64, 64) == _lib.RBN_ERR_INVALID
+
+
 def test_gemv_kernel_time_entry(ctx):
     # the measuring variant launches the same kernel and reports the dispatch's own duration
     M, K, N = 1, 2048, 1024

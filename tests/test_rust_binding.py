@@ -1,0 +1,129 @@
+"""The Rust side of the drop-in is source only (no Rust toolchain in the build image), so it is
+checked as text: the FFI crate declares every entry point of both C headers with the same number
+of parameters in the same order and with matching pointer-ness, its #[repr(C)] structs have the
+headers' fields, and the reference-side patch applies cleanly to the reference checkout when that
+is present."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SYS = os.path.join(ROOT, "rust", "ronn-bitnet-hip-sys", "src", "lib.rs")
+HEADERS = [("rbn", os.path.join(ROOT, "include", "ronn_bitnet_hip.h")),
+           ("rbp", os.path.join(ROOT, "include", "ronn_bitnet_provider.h"))]
+
+
+def c_declarations(path, prefix):
+    text = re.sub(r"/\*.*?\*/", "", open(path).read(), flags=re.S)
+    text = re.sub(r"^\s*#.*$", "", text, flags=re.M)
+    out = {}
+    for m in re.finditer(r"\b(%s_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;" % prefix, text, re.S):
+        args = " ".join(m.group(2).split())
+        params = [] if args == "void" else [a.strip() for a in args.split(",")]
+        out[m.group(1)] = params
+    return out
+
+
+def rust_declarations(path):
+    text = re.sub(r"//.*", "", open(path).read())
+    out = {}
+    for m in re.finditer(r"pub fn (rb[np]_[a-z0-9_]+)\s*\(([^)]*)\)", text, re.S):
+        params = [p.strip() for p in m.group(2).split(",") if p.strip()]
+        out[m.group(1)] = params
+    return out
+
+
+def test_sys_crate_declares_every_entry_point_with_the_same_arity():
+    rust = rust_declarations(SYS)
+    declared = {}
+    for prefix, path in HEADERS:
+        declared.update(c_declarations(path, prefix))
+    assert len(declared) >= 85
+    missing = sorted(set(declared) - set(rust))
+    extra = sorted(set(rust) - set(declared) - {"rbn_last_error", "rbp_last_error"})
+    assert not missing, "not bound in lib.rs: %s" % missing
+    assert not extra, "bound in lib.rs but not in the headers: %s" % extra
+    for name, c_params in declared.items():
+        r_params = rust[name]
+        assert len(c_params) == len(r_params), (name, c_params, r_params)
+        for c, r in zip(c_params, r_params):
+            c_name = re.search(r"([A-Za-z_][A-Za-z_0-9]*)(\s*\[\d+\])?$", c).group(1)
+            r_name, r_type = [x.strip() for x in r.split(":", 1)]
+            assert r_name == c_name, (name, c, r)
+            is_ptr = "*" in c or "[" in c
+            assert is_ptr == r_type.startswith("*"), (name, c, r)
+            if is_ptr and "[" not in c:
+                # constness of the outermost pointee
+                c_const = bool(re.search(r"const\s+\w+\s*\*\s*(const\s*\*)?\s*\w+$", c)) and not re.search(r"\*\s*\*", c)
+                if c.count("*") == 1:
+                    assert r_type.startswith("*const") == c_const, (name, c, r)
+            if not is_ptr:
+                scalar = {"int": "c_int", "float": "f32", "double": "f64", "uint64_t": "u64", "int64_t": "i64",
+                          "size_t": "usize", "uint32_t": "u32", "int32_t": "i32"}
+                assert r_type == scalar[c.split()[-2] if len(c.split()) > 1 else c], (name, c, r)
+
+
+def c_struct_fields(path, name):
+    text = re.sub(r"/\*.*?\*/", "", open(path).read(), flags=re.S)
+    body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (name, name), text, re.S).group(1)
+    return [re.search(r"([A-Za-z_][A-Za-z_0-9]*)\s*(\[\d+\])?$", f.strip()).group(1)
+            for f in body.split(";") if f.strip()]
+
+
+def rust_struct_fields(name):
+    text = re.sub(r"//.*", "", open(SYS).read())
+    m = re.search(r"#\[repr\(C\)\][^{}]*pub struct %s \{(.*?)\}" % name, text, re.S)
+    return [f.split(":")[0].replace("pub", "").strip() for f in m.group(1).split(",") if f.strip()]
+
+
+@pytest.mark.parametrize("header,name", [(0, "rbn_device_info"), (0, "rbn_gemv_problem"), (1, "rbp_config")])
+def test_repr_c_structs_have_the_headers_fields(header, name):
+    assert rust_struct_fields(name) == c_struct_fields(HEADERS[header][1], name)
+
+
+def test_constants_agree_with_the_headers():
+    header = open(HEADERS[0][1]).read()
+    rust = open(SYS).read()
+    for macro in ("RBN_GEMV_MAX_M", "RBN_SKINNY_MAX_M", "RBN_GEMV_GROUP_MAX", "RBN_STATIC_SCRATCH_TILES",
+                  "RBN_KERNEL_GEMV", "RBN_KERNEL_SKINNY", "RBN_KERNEL_MFMA"):
+        c_val = re.search(r"#define %s (\d+)" % macro, header).group(1)
+        r_val = re.search(r"pub const %s: \w+ = (\d+);" % macro, rust).group(1)
+        assert c_val == r_val, macro
+    for name, val in re.findall(r"(RBN_(?:OK|ERR_[A-Z_]+)) = (-?\d+)", header):
+        assert re.search(r"pub const %s: c_int = %s;" % (name, val), rust), name
+
+
+def test_provider_crate_uses_only_bound_symbols():
+    bound = set(rust_declarations(SYS))
+    for f in ("hip_kernel.rs", "provider.rs"):
+        text = open(os.path.join(ROOT, "rust", "ronn-providers-bitnet-hip", "src", f)).read()
+        used = set(re.findall(r"sys::(rb[np]_[a-z0-9_]+)\s*\(", text))
+        assert used and used <= bound, (f, used - bound)
+        # the traits of crates/ronn-core/src/types.rs:153-213,294-303 are implemented in full
+    prov = open(os.path.join(ROOT, "rust", "ronn-providers-bitnet-hip", "src", "provider.rs")).read()
+    for method in ("provider_id", "get_capability", "can_handle", "compile_subgraph", "get_allocator", "configure",
+                   "shutdown", "allocate", "deallocate", "get_memory_info"):
+        assert re.search(r"fn %s\(" % method, prov), method
+    kern = open(os.path.join(ROOT, "rust", "ronn-providers-bitnet-hip", "src", "hip_kernel.rs")).read()
+    for method in ("execute", "get_memory_usage", "get_performance_stats"):
+        assert re.search(r"fn %s\(" % method, kern), method
+
+
+def test_reference_patch_applies(tmp_path):
+    ref = "/root/reference"
+    patch = os.path.join(ROOT, "rust", "patches", "route-matmul-gemm-to-bitnet-provider.patch")
+    files = re.findall(r"^\+\+\+ b/(\S+)", open(patch).read(), flags=re.M)
+    assert len(files) == 5
+    if not os.path.isdir(ref) or shutil.which("patch") is None:
+        pytest.skip("the reference checkout (or patch) is not present on this machine")
+    for f in files:
+        os.makedirs(os.path.dirname(tmp_path / f), exist_ok=True)
+        shutil.copy(os.path.join(ref, f), tmp_path / f)
+    r = subprocess.run(["patch", "-p1", "-i", patch], cwd=tmp_path, capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    session = open(tmp_path / "crates/ronn-api/src/session.rs").read()
+    assert "run_on_provider" in session and "kernel_cache" in session
+    assert "GemmOp" in open(tmp_path / "crates/ronn-onnx/src/ops/mod.rs").read()

@@ -191,12 +191,11 @@ int rbn_act_quant_ternary(rbn_ctx *ctx, const float *d_x, uint64_t M, uint64_t K
     RBN_REQUIRE(M > 0 && K > 0, "M and K must be positive");
     RBN_REQUIRE(d_x && d_q && d_act_scale && d_rowsum, "null pointer in rbn_act_quant_ternary");
     RBN_REQUIRE(M <= 0x7fffffffull, "too many rows");
+    RBN_CHECK(rbn_refuse_while_capturing(ctx, "rbn_act_quant_ternary"));
     const uint64_t n = M * K;
-    // Temporary "packed" image of the activation tensor.
+    // "Packed" image of the activation tensor, in a buffer the context keeps (it only grows).
     void *d_tmp = nullptr;
-    hipError_t e = hipMalloc(&d_tmp, rbn_packed_capacity(n));
-    if (e != hipSuccess)
-        return rbn_fail(RBN_ERR_OOM, "temporary activation buffer: %s", hipGetErrorString(e));
+    RBN_CHECK(rbn_workspace2(ctx, rbn_packed_capacity(n), &d_tmp));
     float scale = 1.0f, thr = 0.0f;
     int rc = rbn_quantize_ternary(ctx, d_x, n, mode, (uint8_t *)d_tmp, &scale, &thr, nullptr);
     if (rc == RBN_OK)
@@ -206,8 +205,6 @@ int rbn_act_quant_ternary(rbn_ctx *ctx, const float *d_x, uint64_t M, uint64_t K
             d_act_scale, scale, M);
         if (hipGetLastError() != hipSuccess) rc = rbn_fail(RBN_ERR_HIP, "fill kernel launch failed");
     }
-    (void)hipStreamSynchronize(ctx->stream);
-    (void)hipFree(d_tmp);
     if (rc != RBN_OK) return rc;
     if (h_scale) *h_scale = scale;
     if (h_threshold) *h_threshold = thr;

@@ -23,6 +23,10 @@ struct rbn_ctx {
     // state); grown on demand by rbn_workspace().
     void *ws = nullptr;
     size_t ws_bytes = 0;
+    // Second grow-only buffer: the packed image of the activations in rbn_act_quant_ternary
+    // (ws is in use by the sums at the same time).
+    void *ws2 = nullptr;
+    size_t ws2_bytes = 0;
     // Pinned host mailbox for the few scalars that come back from the device.
     void *mailbox = nullptr;
     // Split-k workspace of the matmuls: RBN_SPLITK_TILES partial tiles of 16 x 64 int32
@@ -49,6 +53,11 @@ int rbn_skinny_prepare(int device);
 
 // Ensures ctx->ws has at least `bytes` bytes; returns it through *out.
 int rbn_workspace(rbn_ctx *ctx, size_t bytes, void **out);
+// The same for ctx->ws2.
+int rbn_workspace2(rbn_ctx *ctx, size_t bytes, void **out);
+// RBN_ERR_INVALID with a message naming `what` when the context's stream is being captured
+// (for entry points that synchronise, allocate or return scalars to the host).
+int rbn_refuse_while_capturing(rbn_ctx *ctx, const char *what);
 
 #define RBN_HIP(expr)                                                                      \
     do {                                                                                   \

@@ -49,6 +49,34 @@ int rbn_workspace(rbn_ctx *ctx, size_t bytes, void **out) {
     return RBN_OK;
 }
 
+int rbn_workspace2(rbn_ctx *ctx, size_t bytes, void **out) {
+    if (bytes > ctx->ws2_bytes) {
+        if (ctx->ws2) {
+            RBN_HIP(hipStreamSynchronize(ctx->stream));
+            RBN_HIP(hipFree(ctx->ws2));
+            ctx->ws2 = nullptr;
+            ctx->ws2_bytes = 0;
+        }
+        size_t want = (size_t)round_up_u64(bytes, 1 << 20);
+        hipError_t e = hipMalloc(&ctx->ws2, want);
+        if (e != hipSuccess) {
+            ctx->ws2 = nullptr;
+            return rbn_fail(RBN_ERR_OOM, "workspace allocation of %zu bytes failed: %s", want,
+                            hipGetErrorString(e));
+        }
+        ctx->ws2_bytes = want;
+    }
+    *out = ctx->ws2;
+    return RBN_OK;
+}
+
+int rbn_refuse_while_capturing(rbn_ctx *ctx, const char *what) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(ctx->stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone)
+        return rbn_fail(RBN_ERR_INVALID, "%s synchronises the stream and cannot be captured in a graph", what);
+    return RBN_OK;
+}
+
 extern "C" {
 
 const char *rbn_version(void) { return "ronn-bitnet-hip 0.1 (gfx950)"; }
@@ -115,6 +143,7 @@ int rbn_ctx_destroy(rbn_ctx *ctx) {
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     if (ctx->ws) (void)hipFree(ctx->ws);
+    if (ctx->ws2) (void)hipFree(ctx->ws2);
     if (ctx->mailbox) (void)hipHostFree(ctx->mailbox);
     if (ctx->splitk_partials) (void)hipFree(ctx->splitk_partials);
     if (ctx->splitk_tickets) (void)hipFree(ctx->splitk_tickets);

@@ -630,7 +630,8 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
     }
     // published once the stores have completed (vmcnt(0): this wave's; the barrier:
     // everybody's); then one thread draws the ticket
-    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
         const unsigned ticket = atomicAdd(&tickets[h], 1u);

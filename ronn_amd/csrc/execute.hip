@@ -33,6 +33,7 @@ extern "C" int rbn_execute_ternary_matmul(rbn_ctx *ctx, const float *h_a, const 
     RBN_ENTER(ctx);
     RBN_REQUIRE(h_a && h_b && h_out, "null pointer in rbn_execute_ternary_matmul");
     RBN_REQUIRE(M > 0 && N > 0 && K > 0, "M, N and K must be positive");
+    RBN_CHECK(rbn_refuse_while_capturing(ctx, "rbn_execute_ternary_matmul"));
     DeviceScope scope(ctx);
     float *d_a = nullptr, *d_b = nullptr, *d_out = nullptr, *d_as = nullptr;
     int8_t *d_q = nullptr;

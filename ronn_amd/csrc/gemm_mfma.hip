@@ -314,7 +314,11 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
                     off += kThreads * 8;
                     asm volatile("" : "+v"(off));
                 }
-            __builtin_amdgcn_s_waitcnt(kWaitVm0);
+            // the partial tile is published once its stores are acknowledged: the fence keeps the
+            // compiler from moving them below the wait, the wait covers this wave's stores, the
+            // barrier everybody's
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
             if (tid == 0) {
                 const unsigned ticket = atomicAdd(&tickets[tile], 1u);

@@ -46,6 +46,22 @@ std::string shape_str(const std::vector<size_t> &s) {
     return o.str();
 }
 
+// Second digest of the same bytes, unrelated to hash_floats (byte-wise FNV-1a folded with the
+// position): a cache hit needs both to agree.
+uint64_t check_bytes(const void *data, size_t bytes) {
+    const uint8_t *p = static_cast<const uint8_t *>(data);
+    uint64_t a = 0xcbf29ce484222325ull, b = 0x84222325cbf29ce4ull;
+    size_t i = 0;
+    for (; i + 8 <= bytes; i += 8) {
+        uint64_t x;
+        std::memcpy(&x, p + i, 8);
+        a = (a ^ x) * 0x100000001b3ull;
+        b = (b + x) * 0xff51afd7ed558ccdull + (b >> 31);
+    }
+    for (; i < bytes; ++i) a = (a ^ p[i]) * 0x100000001b3ull;
+    return a ^ (b << 1) ^ bytes;
+}
+
 // 64-bit content hash of a weight tensor (four interleaved multiply-xor lanes).
 uint64_t hash_floats(const std::vector<float> &v, const std::vector<size_t> &shape) {
     const uint64_t kMul = 0x9E3779B97F4A7C15ull;
@@ -182,8 +198,10 @@ Tensor BitNetKernel::execute_ternary_matmul(const Tensor &a, const Tensor &b) {
                                  TensorLayout::RowMajor);
     // weights: ternarise + tile once per distinct content (kernels.rs:278 does it per call)
     bool owned = false;
-    const uint64_t key = cache_weights_ ? hash_floats(b.to_vec(), b.shape()) : 0;
-    CachedWeights w = tiled_weights(key, k, n, nullptr, b.to_vec().data(), 1.0f, &owned);
+    const std::vector<float> bv = b.to_vec();
+    const uint64_t key = cache_weights_ ? hash_floats(bv, b.shape()) : 0;
+    const uint64_t chk = cache_weights_ ? check_bytes(bv.data(), bv.size() * 4) : 0;
+    CachedWeights w = tiled_weights(key, chk, bv.size() * 4, k, n, nullptr, bv.data(), 1.0f, &owned);
     struct Release {
         rbn_ctx *c;
         void *p;
@@ -194,7 +212,8 @@ Tensor BitNetKernel::execute_ternary_matmul(const Tensor &a, const Tensor &b) {
     return multiply(a, m, k, n, w.d_tiled, w.scale);
 }
 
-BitNetKernel::CachedWeights BitNetKernel::tiled_weights(uint64_t key, size_t k, size_t n,
+BitNetKernel::CachedWeights BitNetKernel::tiled_weights(uint64_t key, uint64_t check_digest,
+                                                        size_t source_bytes, size_t k, size_t n,
                                                         const uint8_t *h_packed, const float *h_f32,
                                                         float scale, bool *owned) {
     rbn_ctx *ctx = device_->ctx();
@@ -202,7 +221,17 @@ BitNetKernel::CachedWeights BitNetKernel::tiled_weights(uint64_t key, size_t k, 
     *owned = false;
     if (cache_weights_) {
         auto it = weight_cache_.find(key);
-        if (it != weight_cache_.end()) return it->second;
+        if (it != weight_cache_.end()) {
+            CachedWeights &c = it->second;
+            // the key alone is not trusted: a collision would multiply with another matrix
+            if (c.k == k && c.n == n && c.source_bytes == source_bytes && c.check == check_digest) {
+                c.last_use = ++use_clock_;
+                return c;
+            }
+            check(rbn_free(ctx, c.d_tiled), "rbn_free");
+            cache_bytes_ -= c.bytes;
+            weight_cache_.erase(it);
+        }
     }
     DBuf d_p(ctx, rbn_packed_capacity(k * n));
     DBuf d_t(ctx, rbn_tiled_bytes(k, n));
@@ -222,6 +251,22 @@ BitNetKernel::CachedWeights BitNetKernel::tiled_weights(uint64_t key, size_t k, 
     check(rbn_sync(ctx), "rbn_sync");
     w.bytes = rbn_tiled_bytes(k, n);
     w.d_tiled = d_t.release();
+    w.k = k;
+    w.n = n;
+    w.source_bytes = source_bytes;
+    w.check = check_digest;
+    w.last_use = ++use_clock_;
+    // make room: the least recently used matrices go first (every caller holds the kernel's
+    // lock for the whole call, so nothing evicted here is in use)
+    while (cache_weights_ && w.bytes <= max_cache_bytes_ && cache_bytes_ + w.bytes > max_cache_bytes_ &&
+           !weight_cache_.empty()) {
+        auto oldest = weight_cache_.begin();
+        for (auto it = weight_cache_.begin(); it != weight_cache_.end(); ++it)
+            if (it->second.last_use < oldest->second.last_use) oldest = it;
+        check(rbn_free(ctx, oldest->second.d_tiled), "rbn_free");
+        cache_bytes_ -= oldest->second.bytes;
+        weight_cache_.erase(oldest);
+    }
     if (cache_weights_ && cache_bytes_ + w.bytes <= max_cache_bytes_) {
         weight_cache_[key] = w;
         cache_bytes_ += w.bytes;
@@ -277,15 +322,17 @@ Tensor BitNetKernel::execute_prepacked(const Tensor &a, const TernaryTensor &w) 
         return Tensor::from_data(std::vector<float>(m * n, 0.0f), {m, n}, DataType::F32,
                                  TensorLayout::RowMajor);
     // cache key: content of the packed bytes, shape and scale
-    uint64_t key = 0;
+    uint64_t key = 0, chk = 0;
     if (cache_weights_) {
         std::vector<float> as_f((w.packed_data.size() + 3) / 4 + 1, 0.0f);
         std::memcpy(as_f.data(), w.packed_data.data(), w.packed_data.size());
         std::memcpy(&as_f.back(), &w.scale, 4);
         key = hash_floats(as_f, w.shape) ^ 0x5bd1e9955bd1e995ull;
+        chk = check_bytes(as_f.data(), as_f.size() * 4);
     }
     bool owned = false;
-    CachedWeights cw = tiled_weights(key, k, n, w.packed_data.data(), nullptr, w.scale, &owned);
+    CachedWeights cw = tiled_weights(key, chk, w.packed_data.size(), k, n, w.packed_data.data(), nullptr, w.scale,
+                                     &owned);
     struct Release {
         rbn_ctx *c;
         void *p;

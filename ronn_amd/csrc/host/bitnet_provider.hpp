@@ -127,13 +127,18 @@ class BitNetKernel : public CompiledKernel {
         void *d_tiled = nullptr;
         float scale = 1.0f;
         size_t bytes = 0;
+        // what a hit is confirmed with, besides the 64-bit key: dimensions, byte count of the
+        // source and a second, independently computed digest of it
+        size_t k = 0, n = 0, source_bytes = 0;
+        uint64_t check = 0;
+        uint64_t last_use = 0;  // for least-recently-used eviction
     };
     Tensor execute_ternary_matmul(const Tensor &a, const Tensor &b);
     // the shared tail: quantise A, multiply, download
     Tensor multiply(const Tensor &a, size_t m, size_t k, size_t n, const void *d_tiled, float w_scale);
     // tiled device copy of packed weights, cached by `key` when caching is on; *owned tells
     // the caller to free it
-    CachedWeights tiled_weights(uint64_t key, size_t k, size_t n, const uint8_t *h_packed,
+    CachedWeights tiled_weights(uint64_t key, uint64_t check, size_t source_bytes, size_t k, size_t n, const uint8_t *h_packed,
                                 const float *h_f32, float scale, bool *owned);
     void update_stats(double us);  // kernels.rs:235-251
 
@@ -149,6 +154,7 @@ class BitNetKernel : public CompiledKernel {
     MemoryUsage memory_usage_;
     std::unordered_map<uint64_t, CachedWeights> weight_cache_;
     size_t cache_bytes_ = 0;
+    uint64_t use_clock_ = 0;
 };
 
 // kernels.rs:339-344.  Explicit dimensions are checked against the inputs exactly as

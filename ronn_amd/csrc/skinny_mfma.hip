@@ -242,7 +242,7 @@ __global__ __launch_bounds__(MAXW * 64) void skinny_t2_i8_kernel(
     // wave's (a store leaves the counter when the memory system has acknowledged it), the
     // barrier for everybody's; then one thread draws.
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
         const unsigned ticket = atomicAdd(&tickets[group], 1u);

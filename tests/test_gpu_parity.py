@@ -611,6 +611,30 @@ def test_error_paths(ctx):
     assert ctx.lib.rbn_sync(None) == _lib.RBN_ERR_INVALID
 
 
+def test_synchronising_entry_points_refuse_a_capturing_stream(ctx):
+    x = synth_normal(3, 1.0, (4, 64))
+    d_x = ctx.to_device(x)
+    bufs = ctx.alloc_acts(4, 64)
+    ctx.act_quant_ternary(d_x, 4, 64, bufs=bufs)          # sizes the context's buffers beforehand
+    out = np.empty((4, 4), np.float32)
+    ctx.graph_begin()
+    try:
+        with pytest.raises(_lib.RbnError) as e:
+            ctx.act_quant_ternary(d_x, 4, 64, bufs=bufs)
+        assert e.value.code == _lib.RBN_ERR_INVALID and "captured" in e.value.message
+        rc = ctx.lib.rbn_execute_ternary_matmul(ctx.handle, x.ctypes.data, x.T.copy().ctypes.data, 4, 4, 64, 0,
+                                                out.ctypes.data, None)
+        assert rc == _lib.RBN_ERR_INVALID
+        ctx.act_quant_i8(d_x, 4, 64, bufs)                # an asynchronous call is recorded as before
+    finally:
+        g = ctx.graph_end()
+    ctx.graph_launch(g)
+    ctx.sync()
+    ctx.graph_destroy(g)
+    q, s, rs = O.act_quant_i8(x)
+    assert (bufs[0].download(np.int8, 4 * ctx.act_pitch(64)).reshape(4, -1)[:, :64] == q).all()
+
+
 def test_mfma_probe_reports_a_plausible_rate(ctx):
     const = ctx.probe_mfma_i8(0)
     tern = ctx.probe_mfma_i8(1)

@@ -172,6 +172,29 @@ def test_weight_cache_and_stats(provider):
     assert st.execution_count == 4 and st.min_time_us <= st.average_time_us <= st.max_time_us
 
 
+def test_weight_cache_evicts_least_recently_used():
+    # room for two 256 x 128 matrices (8 KiB each, tiled): a third evicts the one not used for longest,
+    # and every product is still right
+    p = create_bitnet_provider_with_config(BitNetProviderConfig(max_cache_size=2 * 256 * 128 // 4))
+    kernel = p.compile_subgraph(matmul_subgraph())
+    a = synth_normal(61, 1.0, (2, 256))
+    ta = Tensor.from_data(a, [2, 256])
+    mats = [synth_normal(70 + i, 0.02, (256, 128)) for i in range(3)]
+
+    def run(i):
+        got = kernel.execute([ta, Tensor.from_data(mats[i], [256, 128])])[0].numpy()
+        assert same_bits(got, O.execute_ternary(a, mats[i])[0]), i
+        return kernel.get_memory_usage()
+
+    assert run(0).allocation_count == 1
+    assert run(1).allocation_count == 2
+    assert run(0).allocation_count == 2                      # hit
+    m = run(2)                                               # evicts matrix 1, not matrix 0
+    assert m.allocation_count == 3 and m.current_bytes == 2 * 256 * 128 // 4
+    assert run(0).allocation_count == 3                      # still cached
+    assert run(1).allocation_count == 4                      # was evicted: rebuilt
+
+
 def test_int8_activation_mode():
     p = create_bitnet_provider_with_config(BitNetProviderConfig(activation="int8"))
     kernel = p.compile_subgraph(matmul_subgraph())

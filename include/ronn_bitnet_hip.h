@@ -244,6 +244,14 @@ int rbn_gemm_t2_i8_skinny(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_sc
 int rbn_gemm_t2_i8_mfma(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,
                         const int32_t *d_rowsum, const uint32_t *d_tiled, float w_scale,
                         uint64_t M, uint64_t K, uint64_t N, int32_t *d_acc, float *d_out);
+/* The launch shape rbn_gemm_t2_i8_skinny picks for a product (needs no device; for tests and
+ * tuning): shape[0] = 1 when the operands travel through a ring in LDS (up to 16 tokens), 0 for
+ * the register ring; [1] workgroups along N; [2] workgroups that share a column group along
+ * k; [3] waves per workgroup; [4] k of one step (64 or 128); [5] steps in all; [6] most steps
+ * any wave gets; [7] bytes of dynamic LDS.  Returns RBN_ERR_UNSUPPORTED for a shape the kernels
+ * would not be launched with (every wave must own at least one step, at most 16 waves, at most
+ * 128 KiB of LDS), RBN_ERR_INVALID for arguments outside the entry point's range. */
+int rbn_skinny_launch_shape(uint64_t M, uint64_t K, uint64_t N, int32_t shape[8]);
 /* rbn_gemm_t2_i8_skinny for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in
  * the reference.  Same arguments, same kernels, same bits; the difference is where narrow

@@ -108,6 +108,7 @@ SIGNATURES = {
                                              C.POINTER(C.c_float)]),
     "rbn_gemv_t2_i8_grouped": (C.c_int, [_vp, C.POINTER(GemvProblem), _u64, _u64, _u64, _u64]),
     "rbn_gemm_t2_i8_skinny": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
+    "rbn_skinny_launch_shape": (C.c_int, [_u64, _u64, _u64, C.POINTER(C.c_int32)]),
     "rbn_gemm_t2_i8_skinny_static": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
     "rbn_gemm_t2_i8_mfma": (C.c_int, [_vp, _vp, _vp, _vp, _vp, C.c_float, _u64, _u64, _u64, _vp, _vp]),
     "rbn_bitlinear_gemv_f32": (C.c_int, [_vp, _vp, _vp, _vp, C.c_float, _vp, C.c_float, _u64, _u64, _vp, _vp]),

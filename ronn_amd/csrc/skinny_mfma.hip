@@ -34,6 +34,7 @@
 //    vmcnt(in flight), never vmcnt(0).
 //  * Weights are code = value + 1; the per-token sum of q is subtracted in the epilogue.
 #include "common.hpp"
+#include <type_traits>
 
 namespace {
 
@@ -338,6 +339,252 @@ int launch_d(hipStream_t stream, const Args &a) {
     }
 }
 
+
+// ---- up to 16 tokens: operands through LDS ------------------------------------------------
+// The MFMA operand layout wants lane l to hold (quad l%16, k-block l/16) of the weights and
+// (token l%16, k-block l/16) of the activations: sixty-four lanes, sixty-four different cache
+// lines.  Loaded straight into registers that way, the texture addresser takes the lanes of a
+// load one by one - measured with cycle counters, each SIMD of a CU got its next wave's
+// eight loads issued ~2200 cycles after the previous wave's, so the sixteenth wave of a
+// workgroup had its data ~8800 cycles after the first and everybody waited for it at the
+// barrier.  Here the loads are global -> LDS transfers (global_load_lds_dwordx4) whose eight
+// consecutive lanes fetch one 128-byte line - a quad's eight k-blocks, a token's 128 k - into a
+// ring that each wave owns; the fragments are then read from LDS in operand order.  The LDS
+// image is the prefill kernel's: unit row*8 + (slot ^ ((row>>1)&7)), which makes the 128-bit
+// reads of sixteen consecutive lanes conflict-free.
+// A stage is 128 k: two loads of weights (quads 0-7, 8-15) and two of activations (tokens
+// 0-7, 8-15), 4 KiB of LDS.  Waves split k as before and never share a stage: no barrier in
+// the loop.  The transfers are issued from inline assembly, so they are counted by hand:
+// before stage d is read, s_waitcnt vmcnt leaves only the stages issued after it in flight.
+
+typedef void __attribute__((address_space(3))) * lds_ptr;
+
+__device__ __forceinline__ void dma16(const void *base, uint32_t lane_offset, uint32_t lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_wave_base), "v"(lane_offset), "s"(base)
+                 : "memory", "m0");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    static_assert(N >= 0 && N < 64, "vmcnt is six bits");
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+constexpr int kStageUnits = 256;  // 16-byte units of one stage: weights 0-127, activations 128-255
+
+template <int D, bool REFILL>
+__global__ __launch_bounds__(1024) void skinny_dma_kernel(
+    const int8_t *__restrict__ q,         // [M][Kpad], Kpad % 128 == 0, M <= 16
+    const float *__restrict__ act_scale, const int32_t *__restrict__ rowsum,
+    const uint4 *__restrict__ wt,         // tiled: uint4 index quad * KB + kb
+    float w_scale, int M, int Kpad, int N, int groups, int splits,
+    int4 *__restrict__ partials, unsigned *__restrict__ tickets,
+    int32_t *__restrict__ acc_out, float *__restrict__ out) {
+    extern __shared__ uint4 ring[];  // [waves][D][kStageUnits]; reused as [waves][256] int4 for the join
+    __shared__ int s_last;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nw = blockDim.x >> 6;
+    const int ql = lane & 15, g = lane >> 4;
+    const int KB = Kpad >> 4;
+    const int stages = Kpad >> 7;  // of 128 k
+    const int group = blockIdx.x % groups, split = blockIdx.x / groups;
+    const int gw = split * nw + wave, gn = splits * nw;
+    const int s0 = gw * stages / gn, s1 = (gw + 1) * stages / gn;  // >= 1 stage (the host sees to it)
+
+    // transfer h of a stage: row (quad or token) 8h + lane/8, slot lane%8 holding k-block
+    // slot ^ ((row>>1)&7) of the stage's eight
+    const int sub = lane >> 3, slot = lane & 7;
+    uint32_t w_off[2], a_off[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int row = 8 * h + sub;
+        const int kb = slot ^ ((row >> 1) & 7);
+        w_off[h] = ((uint32_t)row * (uint32_t)KB + (uint32_t)kb) * 16u;
+        a_off[h] = (uint32_t)min(row, M - 1) * (uint32_t)Kpad + (uint32_t)kb * 16u;
+    }
+    const uint4 *w_base = wt + (size_t)group * 16 * KB;  // the group's sixteen quads exist (N is padded to 64)
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr)ring + (uint32_t)wave * (D * kStageUnits * 16);
+    auto issue = [&](int s, int d) {
+        // past the range: a re-read of the last stage, multiplied by zero (and never below stage 0,
+        // whatever the launch shape: the address must stay inside the matrix)
+        const int sc = max(min(s, s1 - 1), 0);
+        const uint4 *wb = w_base + (size_t)sc * 8;
+        const int8_t *ab = q + (size_t)sc * 128;
+        const uint32_t at = lds0 + (uint32_t)d * (kStageUnits * 16);
+        dma16(wb, w_off[0], at);
+        dma16(wb, w_off[1], at + 1024);
+        dma16(ab, a_off[0], at + 2048);
+        dma16(ab, a_off[1], at + 3072);
+    };
+#pragma unroll
+    for (int d = 0; d < D; ++d) issue(s0 + d, d);
+
+    // fragment positions inside a stage: row ql (quad for the weights, token for the
+    // activations), k-block 4t + g for the two halves t of the stage
+    int f_off[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) f_off[t] = ql * 8 + ((4 * t + g) ^ ((ql >> 1) & 7));
+
+    v4i acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = v4i{0, 0, 0, 0};
+    const uint4 *mine = ring + (size_t)wave * (D * kStageUnits);
+
+    auto consume = [&](int d, uint32_t keep) {
+        const uint4 *st = mine + d * kStageUnits;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const uint4 w = st[f_off[t]];
+            const uint4 a = st[128 + f_off[t]];
+            const v4i af = {(int)(a.x & keep), (int)(a.y & keep), (int)(a.z & keep), (int)(a.w & keep)};
+            acc[0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, decode_b(w.x), acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, decode_b(w.y), acc[1], 0, 0, 0);
+            acc[2] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, decode_b(w.z), acc[2], 0, 0, 0);
+            acc[3] = __builtin_amdgcn_mfma_i32_16x16x64_i8(af, decode_b(w.w), acc[3], 0, 0, 0);
+        }
+    };
+
+    if (!REFILL) {
+        // the ring holds the whole range: stage d has landed when only the 4 (D-1-d) later
+        // transfers are outstanding
+        auto step = [&](auto dt) {
+            constexpr int d = decltype(dt)::value;
+            wait_vm<4 * (D - 1 - d)>();
+            consume(d, s0 + d < s1 ? 0xffffffffu : 0u);
+        };
+        step(std::integral_constant<int, 0>{});
+        if constexpr (D > 1) step(std::integral_constant<int, 1>{});
+        if constexpr (D > 2) step(std::integral_constant<int, 2>{});
+        if constexpr (D > 3) step(std::integral_constant<int, 3>{});
+    } else {
+        // rounds of D stages; stage d is refilled with stage s + D as soon as its fragments are in
+        // registers (lgkmcnt(0): the reads have returned before the transfer may overwrite them)
+        int base = s0;
+        do {
+            auto step = [&](auto dt) {
+                constexpr int d = decltype(dt)::value;
+                wait_vm<4 * (D - 1)>();
+                consume(d, base + d < s1 ? 0xffffffffu : 0u);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                issue(base + d + D, d);
+            };
+            step(std::integral_constant<int, 0>{});
+            if constexpr (D > 1) step(std::integral_constant<int, 1>{});
+            if constexpr (D > 2) step(std::integral_constant<int, 2>{});
+            if constexpr (D > 3) step(std::integral_constant<int, 3>{});
+            base += D;
+        } while (base < s1);
+        wait_vm<0>();  // the last refills (re-reads) must not land on the join below
+    }
+
+    // Join through LDS, each wave writing into its own ring space.  acc[j][i] is token 4*g + i,
+    // column 4*ql + j: one int4 per (token, quad).
+    constexpr int quads = 16, tile = 16 * quads;
+    int4 *red = reinterpret_cast<int4 *>(ring);
+    constexpr int wstride = D * kStageUnits;  // int4 units between two waves' spaces
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        red[wave * wstride + (4 * g + i) * quads + ql] = make_int4(acc[0][i], acc[1][i], acc[2][i], acc[3][i]);
+    __syncthreads();
+
+    const bool vec_ok = (N & 3) == 0;
+    auto finish = [&](int idx, int4 t) {
+        const int row = idx / quads, qd = idx - row * quads;
+        const int col0 = (group * quads + qd) * 4;
+        if (row >= M || col0 >= N) return;
+        const int rs = rowsum[row];
+        const float as = act_scale[row];
+        const int ti[4] = {t.x - rs, t.y - rs, t.z - rs, t.w - rs};
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float f = (float)ti[j] * as;  // kernels.rs:168, left to right
+            v[j] = f * w_scale;
+        }
+        const size_t o = (size_t)row * N + col0;
+        if (vec_ok) {
+            *reinterpret_cast<float4 *>(out + o) = make_float4(v[0], v[1], v[2], v[3]);
+            if (acc_out) *reinterpret_cast<int4 *>(acc_out + o) = make_int4(ti[0], ti[1], ti[2], ti[3]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (col0 + j < N) {
+                    out[o + j] = v[j];
+                    if (acc_out) acc_out[o + j] = ti[j];
+                }
+            }
+        }
+    };
+
+    int4 *my_part = partials + ((size_t)group * splits + split) * tile;
+    for (int idx = tid; idx < tile; idx += blockDim.x) {
+        int4 t = red[idx];
+        for (int w = 1; w < nw; ++w) {
+            const int4 p = red[w * wstride + idx];
+            t.x += p.x;
+            t.y += p.y;
+            t.z += p.z;
+            t.w += p.w;
+        }
+        if (splits == 1)
+            finish(idx, t);
+        else
+            store_device_scope(my_part + idx, t);
+    }
+    if (splits == 1) return;
+
+    // same publication and ticket scheme as skinny_t2_i8_kernel
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned ticket = atomicAdd(&tickets[group], 1u);
+        const int last = ticket == (unsigned)splits - 1;
+        if (last) atomicExch(&tickets[group], 0u);
+        s_last = last;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    const int4 *all = partials + (size_t)group * splits * tile;
+    for (int idx = tid; idx < tile; idx += blockDim.x) {
+        int4 t = make_int4(0, 0, 0, 0);
+        for (int sp0 = 0; sp0 < splits; sp0 += 4) {
+            int4 p[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) p[i] = load_device_scope(all + (size_t)min(sp0 + i, splits - 1) * tile + idx);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int keep = sp0 + i < splits ? -1 : 0;
+                t.x += p[i].x & keep;
+                t.y += p[i].y & keep;
+                t.z += p[i].z & keep;
+                t.w += p[i].w & keep;
+            }
+        }
+        finish(idx, t);
+    }
+}
+
+template <int D, bool REFILL>
+int launch_dma(hipStream_t stream, const Args &a) {
+    const size_t lds = (size_t)a.waves * D * kStageUnits * 16;
+    skinny_dma_kernel<D, REFILL><<<dim3((unsigned)(a.groups * a.splits)), dim3((unsigned)a.waves * 64), lds, stream>>>(
+        a.q, a.act_scale, a.rowsum, a.wt, a.w_scale, a.M, a.Kpad, a.N, a.groups, a.splits, a.partials, a.tickets,
+        a.acc, a.out);
+    return RBN_OK;
+}
+
+template <int D, bool REFILL>
+hipError_t allow_large_lds_dma() {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_dma_kernel<D, REFILL>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+}
+
 }  // namespace
 
 // Scratch of the entry point that allocates nothing (rbn_gemm_t2_i8_skinny_static): partial
@@ -368,6 +615,11 @@ int rbn_skinny_prepare(int device) {
         allow_large_lds<4, 1, 4, false>(), allow_large_lds<4, 1, 4, true>(),
         allow_large_lds<4, 2, 2, false>(), allow_large_lds<4, 2, 2, true>(),
     };
+    const hipError_t results_dma[] = {allow_large_lds_dma<1, false>(), allow_large_lds_dma<2, false>(),
+                                      allow_large_lds_dma<2, true>()};
+    for (hipError_t e : results_dma)
+        if (e != hipSuccess)
+            return rbn_fail(RBN_ERR_HIP, "hipFuncSetAttribute(max dynamic LDS) failed: %s", hipGetErrorString(e));
     for (hipError_t e : results)
         if (e != hipSuccess)
             return rbn_fail(RBN_ERR_HIP, "hipFuncSetAttribute(max dynamic LDS) failed: %s",
@@ -387,6 +639,117 @@ int rbn_skinny_prepare(int device) {
     return RBN_OK;
 }
 
+// The launch shape of a small-batch product: which kernel, how many column groups, how k is split
+// across workgroups and waves.  Pure arithmetic (no device), so the rules can be swept on the CPU.
+struct SkinnyPlan {
+    int mt, ng;       // row tiles of 16 tokens, groups of 64 columns per wave
+    int groups;       // workgroups along N
+    int splits;       // workgroups sharing a column group along k
+    int waves;        // per workgroup
+    int step_k;       // k of one step of a wave's range: 64 (register ring) or 128 (LDS ring)
+    int steps;        // steps in all = Kpad / step_k
+    int longest;      // most steps any wave gets
+    int lds_ring;     // 1: skinny_dma_kernel (up to 16 tokens), 0: skinny_t2_i8_kernel
+    int64_t tiles;    // partial tiles of 16 x 64 int32 the exchange needs (0 without a split)
+    size_t lds_bytes;
+};
+
+// Returns false when `strict` and the exchange does not fit max_tiles / max_groups (the plan then
+// holds what would have been needed); otherwise the split is reduced until it fits.
+static bool plan_skinny(uint64_t M, uint64_t K, uint64_t N, int max_tiles, int max_groups, bool strict,
+                        SkinnyPlan *p) {
+    const int Kpad = (int)rbn_kpad(K);
+    const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
+    // four row tiles and a wide matrix: a wave takes two groups of 64 columns, which halves
+    // the activation traffic (8192 x 28672, M = 64: 55 -> 43 us); narrower matrices need
+    // the workgroups more than the saving (4096 x 11008: 18 us with one group, 28 with two)
+    const int cgroups = (int)(rbn_npad(N) / 64);
+    const int ng = (mt == 4 && cgroups >= 256) ? 2 : 1;
+    const int groups = (cgroups + ng - 1) / ng;
+    // Shape of the launch (measured on the decode shapes; 64-k steps per wave in brackets).
+    // With enough column groups, one workgroup per group: 4096 x 11008 runs 16 waves [4],
+    // 8192 x 28672 16 waves [8].  Narrower matrices are also split along k across
+    // workgroups, towards ~256 of them; the round trip of the partial tiles through
+    // memory costs 1-2 us, which is why wide matrices are not split.  A wave should get 4
+    // steps (a ring of 4 with nothing masked), or 8 and more when the workgroup is full.
+    const int steps = Kpad / 64;
+    const int max_w = mt == 4 ? (ng == 2 ? max_waves<4, 2>() : max_waves<4, 1>())
+                              : (mt == 2 ? max_waves<2, 1>() : max_waves<1, 1>());
+    int splits = 1;
+    if (groups < 128 || groups * max_w < 1024) splits = (256 + groups - 1) / groups;
+    if (splits > steps / 4) splits = steps / 4 > 0 ? steps / 4 : 1;
+    // ... and a split should keep 32 steps or more (48 up to 8 tokens): below that the round
+    // trip of the partial tiles costs more than the extra workgroups bring (2560 x 2560,
+    // M = 4: 8.5 us with 7 splits, 4.5 with one; 4096 x 256: 19 -> 5 us)
+    {
+        const int per = M <= 8 ? 48 : 32;
+        const int want = (steps + per - 1) / per;
+        if (want < splits) splits = want;
+    }
+    // the exchange area holds max_tiles tiles of 16 x 64 int32 and one ticket per group
+    bool fits = true;
+    if (strict) {
+        fits = !(splits > 1 && ((int64_t)groups * splits * mt * ng > max_tiles || groups > max_groups));
+    } else {
+        while (splits > 1 && ((int64_t)groups * splits * mt * ng > max_tiles || groups > max_groups)) --splits;
+    }
+    const int steps_per_split = (steps + splits - 1) / splits;
+    int waves = (steps_per_split + 3) / 4;
+    if (waves > max_w) waves = max_w;
+    if (waves > steps / splits) waves = steps / splits;  // every wave needs a step
+    if (waves < 1) waves = 1;
+    p->mt = mt;
+    p->ng = ng;
+    p->groups = groups;
+    p->lds_ring = mt == 1;
+    p->step_k = 64;
+    p->steps = steps;
+    if (p->lds_ring) {
+        // stages of 128 k; a wave takes about two, every wave at least one
+        const int stages = Kpad / 128;
+        if (splits > stages) splits = stages;
+        const int per_split = (stages + splits - 1) / splits;
+        int w2 = (per_split + 1) / 2;
+        if (w2 > 16) w2 = 16;
+        if (w2 > stages / splits) w2 = stages / splits;
+        if (w2 < 1) w2 = 1;
+        waves = w2;
+        p->step_k = 128;
+        p->steps = stages;
+    }
+    p->splits = splits;
+    p->waves = waves;
+    const int gn = splits * waves;
+    p->longest = (p->steps + gn - 1) / gn;
+    p->tiles = splits > 1 ? (int64_t)groups * splits * mt * ng : 0;
+    p->lds_bytes = p->lds_ring ? (size_t)waves * (p->longest <= 1 ? 1 : 2) * kStageUnits * 16
+                               : (size_t)waves * mt * ng * 16 * 16 * sizeof(int4);
+    return fits;
+}
+
+// What the kernels assume of a launch shape and cannot check themselves.
+static bool plan_is_launchable(const SkinnyPlan &p) {
+    return p.groups >= 1 && p.splits >= 1 && p.waves >= 1 && p.waves <= 16 &&
+           (int64_t)p.splits * p.waves <= p.steps &&  // every wave owns at least one step
+           p.lds_bytes <= 128 * 1024 && (int64_t)p.groups * p.splits < (1ll << 31);
+}
+
+extern "C" int rbn_skinny_launch_shape(uint64_t M, uint64_t K, uint64_t N, int32_t shape[8]) {
+    if (!shape || M == 0 || M > RBN_SKINNY_MAX_M || K == 0 || N == 0 || K > (1ull << 24) || N > (1ull << 24))
+        return RBN_ERR_INVALID;
+    SkinnyPlan p;
+    plan_skinny(M, K, N, RBN_SPLITK_TILES, RBN_SPLITK_GROUPS, false, &p);
+    shape[0] = p.lds_ring;
+    shape[1] = p.groups;
+    shape[2] = p.splits;
+    shape[3] = p.waves;
+    shape[4] = p.step_k;
+    shape[5] = p.steps;
+    shape[6] = p.longest;
+    shape[7] = (int32_t)p.lds_bytes;
+    return plan_is_launchable(p) ? RBN_OK : RBN_ERR_UNSUPPORTED;
+}
+
 // partials / tickets: the split-k exchange area and what it holds (tiles of 4 KiB, counters).
 // With `strict` a launch shape that does not fit is an error; otherwise the split is reduced
 // until it fits (any split gives the same bits).
@@ -403,6 +766,20 @@ static int skinny_impl(rbn_ctx *ctx, const char *name, const int8_t *d_q, const 
     RBN_REQUIRE((((uintptr_t)d_out | (uintptr_t)d_acc) & 15u) == 0,
                 "d_out and d_acc must be 16-byte aligned");
     RBN_REQUIRE(K <= (1ull << 24) && N <= (1ull << 24), "dimension too large");
+    SkinnyPlan p;
+    if (!plan_skinny(M, K, N, max_tiles, max_groups, strict, &p))
+        return rbn_fail(RBN_ERR_UNSUPPORTED,
+                        "%s: M=%llu K=%llu N=%llu needs %lld partial tiles and %d counters; the static "
+                        "scratch holds %d tiles (%zu bytes) and %d counters - use rbn_gemm_t2_i8_skinny",
+                        name, (unsigned long long)M, (unsigned long long)K, (unsigned long long)N,
+                        (long long)p.groups * p.splits * p.mt * p.ng, p.groups, max_tiles, (size_t)max_tiles * 4096,
+                        max_groups);
+    // never launch a shape the kernels do not cover: an index outside a wave's range would be an
+    // address outside the matrix
+    if (!plan_is_launchable(p))
+        return rbn_fail(RBN_ERR_UNSUPPORTED, "%s: no launch shape for M=%llu K=%llu N=%llu (splits %d, waves %d, steps %d)",
+                        name, (unsigned long long)M, (unsigned long long)K, (unsigned long long)N, p.splits, p.waves,
+                        p.steps);
     Args a;
     a.q = d_q;
     a.act_scale = d_act_scale;
@@ -416,62 +793,22 @@ static int skinny_impl(rbn_ctx *ctx, const char *name, const int8_t *d_q, const 
     a.tickets = tickets;
     a.acc = d_acc;
     a.out = d_out;
-    const int mt = M <= 16 ? 1 : M <= 32 ? 2 : 4;
-    // four row tiles and a wide matrix: a wave takes two groups of 64 columns, which halves
-    // the activation traffic (8192 x 28672, M = 64: 55 -> 43 us); narrower matrices need
-    // the workgroups more than the saving (4096 x 11008: 18 us with one group, 28 with two)
-    const int cgroups = (int)(rbn_npad(N) / 64);
-    const int ng = (mt == 4 && cgroups >= 256) ? 2 : 1;
-    a.groups = (cgroups + ng - 1) / ng;
-    // Shape of the launch (measured on the decode shapes; 64-k steps per wave in brackets).
-    // With enough column groups, one workgroup per group: 4096 x 11008 runs 16 waves [4],
-    // 8192 x 28672 16 waves [8].  Narrower matrices are also split along k across
-    // workgroups, towards ~256 of them; the round trip of the partial tiles through
-    // memory costs 1-2 us, which is why wide matrices are not split.  A wave should get 4
-    // steps (a ring of 4 with nothing masked), or 8 and more when the workgroup is full.
-    const int steps = a.Kpad / 64;
-    const int max_w = mt == 4 ? (ng == 2 ? max_waves<4, 2>() : max_waves<4, 1>())
-                              : (mt == 2 ? max_waves<2, 1>() : max_waves<1, 1>());
-    int splits = 1;
-    if (a.groups < 128 || a.groups * max_w < 1024) splits = (256 + a.groups - 1) / a.groups;
-    if (splits > steps / 4) splits = steps / 4 > 0 ? steps / 4 : 1;
-    // ... and a split should keep 32 steps or more (48 up to 8 tokens): below that the round
-    // trip of the partial tiles costs more than the extra workgroups bring (2560 x 2560,
-    // M = 4: 8.5 us with 7 splits, 4.5 with one; 4096 x 256: 19 -> 5 us)
-    {
-        const int per = M <= 8 ? 48 : 32;
-        const int want = (steps + per - 1) / per;
-        if (want < splits) splits = want;
-    }
-    // the exchange area holds max_tiles tiles of 16 x 64 int32 and one ticket per group
-    if (strict) {
-        if (splits > 1 && ((int64_t)a.groups * splits * mt * ng > max_tiles || a.groups > max_groups))
-            return rbn_fail(RBN_ERR_UNSUPPORTED,
-                            "%s: M=%llu K=%llu N=%llu needs %lld partial tiles and %d counters; the static "
-                            "scratch holds %d tiles (%zu bytes) and %d counters - use rbn_gemm_t2_i8_skinny",
-                            name, (unsigned long long)M, (unsigned long long)K, (unsigned long long)N,
-                            (long long)a.groups * splits * mt * ng, a.groups, max_tiles,
-                            (size_t)max_tiles * 4096, max_groups);
-    } else {
-        while (splits > 1 && ((int64_t)a.groups * splits * mt * ng > max_tiles || a.groups > max_groups))
-            --splits;
-    }
-    const int steps_per_split = (steps + splits - 1) / splits;
-    int waves = (steps_per_split + 3) / 4;
-    if (waves > max_w) waves = max_w;
-    if (waves > steps / splits) waves = steps / splits;  // every wave needs a step
-    if (waves < 1) waves = 1;
-    a.splits = splits;
-    a.waves = waves;
-    if (strict && splits > 1) {
+    a.groups = p.groups;
+    a.splits = p.splits;
+    a.waves = p.waves;
+    if (strict && a.splits > 1) {
         // the array keeps the last call's contents: the counters this launch draws from start at zero
         clear_tickets_kernel<<<dim3(1), dim3(kStaticGroups), 0, ctx->stream>>>(tickets, kStaticGroups);
     }
     int rc;
-    switch (mt) {
-        case 1: rc = launch_d<1, 1>(ctx->stream, a); break;
+    switch (p.mt) {
+        case 1:
+            rc = p.longest <= 1 ? launch_dma<1, false>(ctx->stream, a)
+                                : p.longest <= 2 ? launch_dma<2, false>(ctx->stream, a)
+                                                 : launch_dma<2, true>(ctx->stream, a);
+            break;
         case 2: rc = launch_d<2, 1>(ctx->stream, a); break;
-        default: rc = ng == 2 ? launch_d<4, 2>(ctx->stream, a) : launch_d<4, 1>(ctx->stream, a); break;
+        default: rc = p.ng == 2 ? launch_d<4, 2>(ctx->stream, a) : launch_d<4, 1>(ctx->stream, a); break;
     }
     RBN_CHECK(rc);
     RBN_HIP(hipGetLastError());

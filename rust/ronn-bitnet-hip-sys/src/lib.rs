@@ -292,6 +292,7 @@ extern "C" {
         d_acc: *mut i32,
         d_out: *mut f32,
     ) -> c_int;
+    pub fn rbn_skinny_launch_shape(M: u64, K: u64, N: u64, shape: *mut i32) -> c_int;
     pub fn rbn_gemm_t2_i8_skinny_static(
         ctx: *mut rbn_ctx,
         d_q: *const i8,

@@ -235,3 +235,42 @@ def test_packed_weight_file_rejects_damage(lib, tmp_path):
     dirty[-1] |= 0x80
     with pytest.raises(bitnet.Error, match="tail bits"):
         bitnet.TernaryTensor.from_parts(dirty, [5], 1.0, 0.0)
+
+
+def test_small_batch_launch_shapes_meet_the_kernels_assumptions(lib):
+    """The small-batch kernels trust their launch shape: a wave whose share of k were empty would
+    read outside the matrix.  The rule that picks the shape is pure arithmetic, so it is swept
+    here: every wave owns at least one step, no workgroup has more than 16 waves or 128 KiB of
+    LDS, and the steps cover K exactly."""
+    shape = (C.c_int32 * 8)()
+    ks = list(range(1, 300)) + [511, 512, 513, 1000, 2048, 2560, 4096, 6912, 8192, 11008, 12288, 15000,
+                                16384, 28672, 100000, 1 << 20]
+    ns = [1, 3, 37, 64, 65, 130, 256, 1024, 1376, 2560, 4096, 8128, 8192, 11008, 16384, 28672, 32000, 200000]
+    checked = 0
+    for M in (1, 2, 7, 8, 9, 16, 17, 32, 33, 64):
+        for K in ks:
+            for N in ns:
+                rc = lib.rbn_skinny_launch_shape(M, K, N, shape)
+                assert rc == 0, (M, K, N, list(shape))
+                ring, groups, splits, waves, step_k, steps, longest, lds = list(shape)
+                kpad = (K + 127) // 128 * 128
+                assert ring == (1 if M <= 16 else 0) and step_k == (128 if ring else 64)
+                assert steps * step_k == kpad
+                assert 1 <= waves <= 16 and splits >= 1 and splits * waves <= steps
+                assert longest == -(-steps // (splits * waves)) and longest >= 1
+                assert 0 < lds <= 128 * 1024
+                assert groups >= 1 and groups * 64 * (2 if (M > 32 and -(-N // 64) >= 256) else 1) >= N
+                # the partition the kernels use: wave w of g takes steps [w*steps/g, (w+1)*steps/g)
+                g = splits * waves
+                assert all((w + 1) * steps // g > w * steps // g for w in range(g))
+                if splits > 1:
+                    assert groups <= 1024 and groups * splits * -(-M // 16) <= 16384
+                checked += 1
+    assert checked > 50000
+    for bad in ((0, 64, 64), (65, 64, 64), (1, 0, 64), (1, 64, 0)):
+        assert lib.rbn_skinny_launch_shape(*bad, shape) == _lib.RBN_ERR_INVALID
+    # the recorded shapes of the decode sweep
+    lib.rbn_skinny_launch_shape(16, 4096, 11008, shape)
+    assert list(shape)[:7] == [1, 172, 1, 16, 128, 32, 2]
+    lib.rbn_skinny_launch_shape(16, 4096, 4096, shape)
+    assert list(shape)[:4] == [1, 64, 2, 8]

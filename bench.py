@@ -603,6 +603,7 @@ def main():
                                "so every GEMV streams from HBM; HIP-graph replay; the one-GEMV-per-launch figure is "
                                "extra.gemv_one_per_launch" % (GROUP, gw.n, gw.n * gw.tiled_bytes / 2**20),
                    "M": M, "K": K, "N": N, "gemvs_per_launch": GROUP, "weight_buffers": gw.n,
+                   "gemvs_timed": args.steps * GROUP,
                    "preheat": "0.25 s of the same launches during set-up, before the warm-up steps (clock ramp)",
                    "device": info["name"] or info["arch"], "arch": info["arch"],
                    "compute_units": info["compute_units"], "clock_mhz": info["clock_khz"] / 1000.0},

@@ -136,3 +136,128 @@ def test_lds_ring_kernel_model(lib, M, K, N):
     want = q_src.astype(np.int64) @ vals.astype(np.int64)
     rowsum = q.astype(np.int64).sum(axis=1, keepdims=True)
     assert (got - rowsum == want).all()
+
+
+# ---- prefill kernel (gemm_t2_i8_mfma_kernel<2> in ronn_amd/csrc/gemm_mfma.hip), one workgroup ------------
+
+def mfma_32x32x32_i8(a_lane, b_lane):
+    """v_mfma_i32_32x32x32_i8: lane l gives A[row l%32][16 k of half l//32] and B[the same k][column l%32];
+    result register r of lane l is D[8*(r//4) + 4*(l//32) + r%4][l%32]."""
+    A = np.zeros((32, 32), dtype=np.int64)
+    B = np.zeros((32, 32), dtype=np.int64)
+    for l in range(64):
+        A[l % 32, 16 * (l // 32):16 * (l // 32) + 16] = a_lane[l]
+        B[16 * (l // 32):16 * (l // 32) + 16, l % 32] = b_lane[l]
+    D = A @ B
+    out = np.zeros((64, 16), dtype=np.int64)
+    for l in range(64):
+        for r in range(16):
+            out[l, r] = D[8 * (r // 4) + 4 * (l // 32) + r % 4, l % 32]
+    return out
+
+
+@pytest.mark.parametrize("M,K,N,bm,bn", [(128, 256, 256, 0, 0), (200, 384, 300, 1, 1), (130, 128, 260, 1, 0)])
+def test_prefill_tile_model(M, K, N, bm, bn):
+    """One 128 x 256 tile (bm, bn): the stage transfers' source addresses and LDS units, the fragment
+    units every lane reads, the 32 MFMAs per K step and the epilogue's row / column mapping."""
+    rng = np.random.default_rng(M + K + N)
+    vals = rng.integers(-1, 2, size=(K, N)).astype(np.int8)
+    q_src = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    tiled, kpad, npad = tile_weights(vals)
+    KB, nquads = kpad // 16, npad // 4
+    q = np.zeros((M, kpad), dtype=np.int8)
+    q[:, :K] = q_src
+    qbytes = q.reshape(-1).view(np.uint8)
+    TM, BN, BK = 128, 256, 128
+    kA, kB = TM * 8, (BN // 4) * 8           # 16-byte units of an activation / a weight stage
+    m0, n0 = bm * TM, bn * BN
+    q0 = n0 >> 2
+    iters = kpad // BK
+    result = np.zeros((TM, BN), dtype=np.int64)
+    for it in range(iters):
+        # --- issue(): four waves, per wave 4 activation transfers and 2 weight transfers of 64 lanes
+        sa = np.zeros(kA * 16, dtype=np.uint8)
+        sb = np.zeros(kB * 16, dtype=np.uint8)
+        for wave in range(4):
+            for lane in range(64):
+                sub = lane >> 3
+                for j in range(4):
+                    lrow = (4 * j + wave) * 8 + sub
+                    seg = (lane & 7) ^ ((lrow >> 1) & 7)
+                    src = (m0 * kpad + it * BK) + (min(m0 + lrow, M - 1) - m0) * kpad + seg * 16
+                    assert 0 <= src and src + 16 <= qbytes.size
+                    dst = (4 * j + wave) * 1024 + 16 * lane
+                    sa[dst:dst + 16] = qbytes[src:src + 16]
+                for j in range(2):
+                    lquad = (4 * j + wave) * 8 + sub
+                    kb = (lane & 7) ^ ((lquad >> 1) & 7)
+                    src = (q0 * KB + it * (BK // 16)) * 16 + ((min(q0 + lquad, nquads - 1) - q0) * KB + kb) * 16
+                    assert 0 <= src and src + 16 <= tiled.size
+                    dst = (4 * j + wave) * 1024 + 16 * lane
+                    sb[dst:dst + 16] = tiled[src:src + 16]
+        # --- fragments and MFMAs: wave (wm, wn) owns rows wm*64 .. +63, quads wn*32 .. +31
+        for wave in range(4):
+            wm, wn = wave >> 1, wave & 1
+            lanes = np.arange(64)
+            frow0 = wm * 64 + (lanes & 31)
+            khalf = lanes >> 5
+            fquad = wn * 32 + (lanes & 31)
+            acc = np.zeros((2, 4, 64, 16), dtype=np.int64)
+            for ks in range(4):
+                seg = 2 * ks + khalf
+                a_unit = frow0 * 8 + (seg ^ ((frow0 >> 1) & 7))
+                b_unit = fquad * 8 + (seg ^ ((fquad >> 1) & 7))
+                assert a_unit.max() + 32 * 8 < kA and b_unit.max() < kB
+                ra0 = np.stack([sa[16 * u:16 * u + 16].view(np.int8) for u in a_unit]).astype(np.int64)
+                ra1 = np.stack([sa[16 * (u + 256):16 * (u + 256) + 16].view(np.int8) for u in a_unit]).astype(np.int64)
+                rb = np.stack([sb[16 * u:16 * u + 16].view(np.uint32) for u in b_unit])
+                for j in range(4):
+                    bf = np.stack([decode_b(int(rb[l, j])) for l in range(64)])
+                    acc[0, j] += mfma_32x32x32_i8(ra0, bf)
+                    acc[1, j] += mfma_32x32x32_i8(ra1, bf)
+            # --- epilogue mapping: lane owns columns 4*fquad + j, rows wm*64 + mt*32 + 8*(r//4) + 4*(lane//32) + r%4
+            for mt in range(2):
+                for j in range(4):
+                    for l in range(64):
+                        for r in range(16):
+                            lrow = wm * 64 + mt * 32 + 8 * (r >> 2) + 4 * (l >> 5) + (r & 3)
+                            result[lrow, fquad[l] * 4 + j] += acc[mt, j, l, r]
+    rows = min(TM, M - m0)
+    cols = min(BN, N - n0)
+    rowsum = q.astype(np.int64).sum(axis=1)[m0:m0 + rows, None]
+    want = (q_src.astype(np.int64) @ vals.astype(np.int64))[m0:m0 + rows, n0:n0 + cols]
+    assert (result[:rows, :cols] - rowsum == want).all()
+
+
+# ---- decode GEMV (gemv.hip): the 4-bit planes that feed v_dot8 ---------------------------------------------
+
+def test_gemv_nibble_planes_reproduce_the_int8_dot_product():
+    """to_nibble_planes() and the even / odd 2-bit fields of a tiled weight word: an int8 activation is
+    16 * hi + lo (hi a signed, lo an unsigned nibble); (w & 0x33333333) and ((w >> 2) & 0x33333333) are
+    the codes of k = (0,8,1,9,2,10,3,11) and (4,12,5,13,6,14,7,15) as nibbles, the order the planes are
+    packed in, so that 16 * (sdot8 + sdot8) + (udot8 + udot8) is the dot product with the 16 codes."""
+    rng = np.random.default_rng(5)
+    for _ in range(200):
+        a = rng.integers(-128, 128, size=16).astype(np.int8)
+        code = rng.integers(0, 3, size=16).astype(np.uint32)
+        w = np.uint32(0)
+        for k in range(16):
+            s, b = k // 4, k % 4
+            w |= np.uint32(int(code[k]) << (8 * b + 2 * s))
+        ax, ay, az, aw = (int(x) for x in a.view(np.uint32))
+        px = ((ax >> 4) & 0x0F0F0F0F) | (az & 0xF0F0F0F0)
+        py = (ax & 0x0F0F0F0F) | ((az & 0x0F0F0F0F) << 4)
+        pz = ((ay >> 4) & 0x0F0F0F0F) | (aw & 0xF0F0F0F0)
+        pw = (ay & 0x0F0F0F0F) | ((aw & 0x0F0F0F0F) << 4)
+        ev, od = int(w) & 0x33333333, (int(w) >> 2) & 0x33333333
+
+        def nibbles(x, signed):
+            out = [(x >> (4 * i)) & 15 for i in range(8)]
+            return [n - 16 if signed and n >= 8 else n for n in out]
+
+        def dot8(x, y, signed):
+            return sum(p * q for p, q in zip(nibbles(x, signed), nibbles(y, signed)))
+
+        hi = dot8(px, ev, True) + dot8(pz, od, True)
+        lo = dot8(py, ev, False) + dot8(pw, od, False)
+        assert 16 * hi + lo == int((a.astype(np.int64) * code.astype(np.int64)).sum())

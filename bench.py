@@ -529,6 +529,30 @@ def profile_kernel(ctx, which, launches):
     elif which == "stream":
         print(json.dumps(time_stream_floor(ctx)))
         return
+    elif which == "skinny_trace":
+        # needs a library built with the cycle stamps: make -B -C ronn_amd/csrc EXTRA=-DRBN_SK_TRACE
+        fn = getattr(ctx.lib, "rbn_debug_sk_trace", None)
+        if fn is None:
+            print("bench.py: this library has no cycle stamps; rebuild with "
+                  "`make -B -C ronn_amd/csrc EXTRA=-DRBN_SK_TRACE`", file=sys.stderr)
+            sys.exit(2)
+        fn.argtypes, fn.restype = [C.c_void_p, C.c_int], C.c_int
+        wl = Workload(ctx, 16, 4096, 11008, 0.02, seed=3, mode=1)
+        for i in range(40):
+            wl.launch(ctx.skinny, i)
+        ctx.sync()
+        wl.launch(ctx.skinny, 17)
+        ctx.sync()
+        buf = np.zeros(64 * 16 * 8, dtype=np.int64)
+        _lib.check(fn(buf.ctypes.data, buf.size))
+        t = buf.reshape(64, 16, 8)[:, :, :5]
+        t = t - t[:, :, 0:1].min(axis=1, keepdims=True)      # cycles since the workgroup's first wave started
+        names = ["start", "transfers_issued", "last_mfma_done", "past_join_barrier", "stores_acknowledged"]
+        print(json.dumps({"kernel": "skinny_dma_kernel", "M": 16, "K": 4096, "N": 11008, "unit": "shader clock cycles",
+                          "workgroup_0": {n: [int(v) for v in t[0, :, i]] for i, n in enumerate(names)},
+                          "median_over_64_workgroups_of_the_slowest_wave": {
+                              n: float(np.median(t[:, :, i].max(axis=1))) for i, n in enumerate(names)}}))
+        return
     elif which in ("decoder", "decoder_eager"):
         # decoder_eager launches kernel by kernel instead of replaying the captured graph
         # (for per-kernel traces)
@@ -552,7 +576,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="headline only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline timings (parity is still gated)")
     ap.add_argument("--kernel", choices=["gemv_grouped", "gemv", "skinny", "gemm", "pack", "quantize", "copy",
-                                         "act_quant", "stream", "decoder", "decoder_eager"],
+                                         "act_quant", "stream", "skinny_trace", "decoder", "decoder_eager"],
                     help="profiling aid: launch only this kernel a few times (for rocprofv3) and exit")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -36,6 +36,27 @@
 #include "common.hpp"
 #include <type_traits>
 
+// Optional cycle stamps (built only with -DRBN_SK_TRACE, e.g. `make -B EXTRA=-DRBN_SK_TRACE`): every wave of
+// the first 64 workgroups of skinny_dma_kernel records the shader clock at five points - kernel start,
+// transfers issued, last MFMA done, past the join barrier, stores acknowledged - and
+// rbn_debug_sk_trace copies the stamps to the host.  `python3 bench.py --kernel skinny_trace` prints them.
+#ifdef RBN_SK_TRACE
+__device__ long long g_sk_trace[64 * 16 * 8];
+#define SK_STAMP(i)                                                                                      \
+    do {                                                                                                 \
+        if ((threadIdx.x & 63) == 0 && blockIdx.x < 64)                                                  \
+            g_sk_trace[(blockIdx.x * 16 + (threadIdx.x >> 6)) * 8 + (i)] = (long long)__builtin_readcyclecounter(); \
+    } while (0)
+extern "C" int rbn_debug_sk_trace(long long *h_out, int count) {
+    if (!h_out || count < 0 || count > 64 * 16 * 8) return RBN_ERR_INVALID;
+    return hipMemcpyFromSymbol(h_out, HIP_SYMBOL(g_sk_trace), sizeof(long long) * (size_t)count) == hipSuccess
+               ? RBN_OK
+               : RBN_ERR_HIP;
+}
+#else
+#define SK_STAMP(i)
+#endif
+
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -385,6 +406,7 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
     extern __shared__ uint4 ring[];  // [waves][D][kStageUnits]; reused as [waves][256] int4 for the join
     __shared__ int s_last;
 
+    SK_STAMP(0);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -423,6 +445,7 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
     };
 #pragma unroll
     for (int d = 0; d < D; ++d) issue(s0 + d, d);
+    SK_STAMP(1);
 
     // fragment positions inside a stage: row ql (quad for the weights, token for the
     // activations), k-block 4t + g for the two halves t of the stage
@@ -482,6 +505,7 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
         wait_vm<0>();  // the last refills (re-reads) must not land on the join below
     }
 
+    SK_STAMP(2);
     // Join through LDS, each wave writing into its own ring space.  acc[j][i] is token 4*g + i,
     // column 4*ql + j: one int4 per (token, quad).
     constexpr int quads = 16, tile = 16 * quads;
@@ -491,6 +515,7 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
     for (int i = 0; i < 4; ++i)
         red[wave * wstride + (4 * g + i) * quads + ql] = make_int4(acc[0][i], acc[1][i], acc[2][i], acc[3][i]);
     __syncthreads();
+    SK_STAMP(3);
 
     const bool vec_ok = (N & 3) == 0;
     auto finish = [&](int idx, int4 t) {
@@ -536,7 +561,13 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
         else
             store_device_scope(my_part + idx, t);
     }
-    if (splits == 1) return;
+    if (splits == 1) {
+#ifdef RBN_SK_TRACE
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        SK_STAMP(4);
+#endif
+        return;
+    }
 
     // same publication and ticket scheme as skinny_t2_i8_kernel
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");

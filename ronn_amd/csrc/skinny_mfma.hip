@@ -143,7 +143,7 @@ __global__ __launch_bounds__(MAXW * 64) void skinny_t2_i8_kernel(
     uint4 wr[D][NG], ar[D][MT];
 #pragma unroll
     for (int d = 0; d < D; ++d) {
-        const int s = min(s0 + d, s1 - 1);
+        const int s = max(min(s0 + d, s1 - 1), 0);  // never below step 0, whatever the launch shape
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) ar[d][mt] = ap[mt][4 * s];
 #pragma unroll
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(MAXW * 64) void skinny_t2_i8_kernel(
                                    ar[d][mt].w & keep);
             consume(wr[d], a);
             if (REFILL) {
-                const int sn = min(base + d + D, s1 - 1);
+                const int sn = max(min(base + d + D, s1 - 1), 0);
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) ar[d][mt] = ap[mt][4 * sn];
 #pragma unroll

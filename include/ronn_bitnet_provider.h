@@ -80,6 +80,20 @@ int rbp_kernel_destroy(rbp_kernel *k);
 int rbp_kernel_execute(rbp_kernel *k, int n_inputs, const float *const *h_data,
                        const uint64_t *const *shapes, const int *ndims, const int *dtypes,
                        float *h_out, uint64_t out_capacity, uint64_t out_shape[2]);
+/* Several independent TernaryMatMul nodes of one shape in one call: n_pairs pairs
+ * (A_i [m,k], B_i [k,n]), host f32 buffers; h_out[i] (capacity out_capacity_each elements)
+ * receives what rbp_kernel_execute gives for {A_i, B_i}, bit for bit.  The reference runs such
+ * nodes one execute() at a time (kernels.rs:254-319, issued per node by
+ * ProviderRegistry::compile_subgraph, registry.rs:237-266); here the nodes a graph holds side
+ * by side (q/k/v or gate/up projections of one token, one layer of several sequences) share
+ * one launch in the decode regime (rbn_gemv_t2_i8_grouped, up to RBN_GEMV_GROUP_MAX per
+ * launch); nodes that pass the same A are quantised once.  *launches (optional) receives the
+ * number of matmul launches issued.  Errors as rbp_kernel_execute, plus a message naming the
+ * node whose shape differs from node 0's. */
+int rbp_kernel_execute_group(rbp_kernel *k, int n_pairs, const float *const *h_a,
+                             const float *const *h_b, const uint64_t shape_a[2],
+                             const uint64_t shape_b[2], float *const *h_out,
+                             uint64_t out_capacity_each, int *launches);
 /* get_performance_stats / get_memory_usage (kernels.rs:321-327). */
 int rbp_kernel_stats(rbp_kernel *k, uint64_t *execution_count, double *average_us, double *min_us,
                      double *max_us);

@@ -240,6 +240,7 @@ PROVIDER_SIGNATURES = {
     "rbp_ternary_save": (C.c_int, [_vp, C.c_char_p]),
     "rbp_ternary_load": (C.c_int, [C.c_char_p, C.POINTER(_vp)]),
     "rbp_kernel_execute_prepacked": (C.c_int, [_vp, _vp, _u64p, C.c_int, _vp, _vp, _u64, _u64p]),
+    "rbp_kernel_execute_group": (C.c_int, [_vp, C.c_int, _vp, _vp, _u64p, _u64p, _vp, _u64, C.POINTER(C.c_int)]),
 }
 
 _bound = None
@@ -370,6 +371,40 @@ class BitNetKernel:
                                          cap, out_shape))
         m, nn = out_shape[0], out_shape[1]
         return [Tensor(out[:m * nn].reshape(m, nn), DataType.F32, TensorLayout.RowMajor)]
+
+    def execute_group(self, inputs: Sequence[Tensor]) -> List[Tensor]:
+        """Several independent TernaryMatMul nodes of one shape, passed as the pairs
+        (A_0, B_0, A_1, B_1, ...): result i is what execute([A_i, B_i]) returns.  In the decode
+        regime the nodes share one GPU launch; `last_group_launches` holds the number of
+        matmul launches the call issued."""
+        if len(inputs) == 0 or len(inputs) % 2:
+            raise Error("Ternary MatMul group requires pairs of inputs (A_i, B_i)")
+        for t in inputs:
+            if t.dtype() != DataType.F32:
+                raise Error("BitNet quantization requires FP32 input tensors")
+        n = len(inputs) // 2
+        a0, b0 = inputs[0], inputs[1]
+        if len(a0.shape()) != 2 or len(b0.shape()) != 2:
+            raise Error("Matrix dimension mismatch: A=%s, B=%s, expected A=[m,k], B=[k,n]"
+                        % (a0.shape(), b0.shape()))
+        for i in range(1, n):
+            # the C entry point takes one shape for the whole group, so this is checked here
+            if inputs[2 * i].shape() != a0.shape() or inputs[2 * i + 1].shape() != b0.shape():
+                raise Error("Ternary MatMul group: node %d has A=%s, B=%s, the group's shape is A=%s, B=%s"
+                            % (i, inputs[2 * i].shape(), inputs[2 * i + 1].shape(), a0.shape(), b0.shape()))
+        a_arr = [np.ascontiguousarray(inputs[2 * i].to_vec(), dtype=np.float32) for i in range(n)]
+        b_arr = [np.ascontiguousarray(inputs[2 * i + 1].to_vec(), dtype=np.float32) for i in range(n)]
+        m, nn = a0.shape()[0], b0.shape()[1]
+        cap = max(1, m * nn)
+        outs = [np.empty(cap, dtype=np.float32) for _ in range(n)]
+        pa = (_vp * n)(*[x.ctypes.data for x in a_arr])
+        pb = (_vp * n)(*[x.ctypes.data for x in b_arr])
+        po = (_vp * n)(*[x.ctypes.data for x in outs])
+        launches = C.c_int(0)
+        _check(_api().rbp_kernel_execute_group(self._h, n, pa, pb, _shape_arg(a0.shape()), _shape_arg(b0.shape()),
+                                               po, cap, C.byref(launches)))
+        self.last_group_launches = launches.value
+        return [Tensor(o[:m * nn].reshape(m, nn), DataType.F32, TensorLayout.RowMajor) for o in outs]
 
     def execute_prepacked(self, a: Tensor, weights: "TernaryTensor") -> Tensor:
         """TernaryMatMul with weights that are already ternarised (a loaded weight file)."""

@@ -260,9 +260,12 @@ BitNetKernel::CachedWeights BitNetKernel::tiled_weights(uint64_t key, uint64_t c
     // lock for the whole call, so nothing evicted here is in use)
     while (cache_weights_ && w.bytes <= max_cache_bytes_ && cache_bytes_ + w.bytes > max_cache_bytes_ &&
            !weight_cache_.empty()) {
-        auto oldest = weight_cache_.begin();
+        auto oldest = weight_cache_.end();
         for (auto it = weight_cache_.begin(); it != weight_cache_.end(); ++it)
-            if (it->second.last_use < oldest->second.last_use) oldest = it;
+            if (!pinned_.count(it->first) &&
+                (oldest == weight_cache_.end() || it->second.last_use < oldest->second.last_use))
+                oldest = it;
+        if (oldest == weight_cache_.end()) break;  // everything left is in use by this call
         check(rbn_free(ctx, oldest->second.d_tiled), "rbn_free");
         cache_bytes_ -= oldest->second.bytes;
         weight_cache_.erase(oldest);
@@ -302,6 +305,145 @@ Tensor BitNetKernel::multiply(const Tensor &a, size_t m, size_t k, size_t n, con
     std::vector<float> result(m * n);
     check(rbn_d2h(ctx, result.data(), d_o.p, m * n * 4), "rbn_d2h");
     return Tensor::from_data(std::move(result), {m, n}, DataType::F32, TensorLayout::RowMajor);
+}
+
+std::vector<Tensor> BitNetKernel::execute_group(const std::vector<Tensor> &inputs, int *launches) {
+    const auto start = std::chrono::steady_clock::now();
+    std::lock_guard<std::mutex> guard(lock_);
+    if (launches) *launches = 0;
+    if (operation_.kind != BitNetOperation::TernaryMatMul)
+        throw Error("execute_group needs a TernaryMatMul kernel");
+    if (inputs.empty() || inputs.size() % 2 != 0)
+        throw Error("Ternary MatMul group requires pairs of inputs (A_i, B_i)");
+    const size_t count = inputs.size() / 2;
+    // every node is checked as execute() checks it (kernels.rs:142-152, quantization.rs:68-72)
+    const Tensor &a0 = inputs[0], &b0 = inputs[1];
+    for (const Tensor &t : inputs) require_f32(t);
+    if (a0.shape().size() != 2 || b0.shape().size() != 2 || a0.shape()[1] != b0.shape()[0])
+        throw Error("Matrix dimension mismatch: A=" + shape_str(a0.shape()) + ", B=" + shape_str(b0.shape()) +
+                    ", expected A=[m,k], B=[k,n]");
+    const size_t m = a0.shape()[0], k = a0.shape()[1], n = b0.shape()[1];
+    if ((operation_.m || operation_.n || operation_.k) &&
+        (operation_.m != m || operation_.n != n || operation_.k != k)) {
+        std::ostringstream o;
+        o << "Matrix dimension mismatch: A=" << shape_str(a0.shape()) << ", B=" << shape_str(b0.shape())
+          << ", expected A=[" << operation_.m << "," << operation_.k << "], B=[" << operation_.k << ","
+          << operation_.n << "]";
+        throw Error(o.str());
+    }
+    for (size_t i = 1; i < count; ++i)
+        if (inputs[2 * i].shape() != a0.shape() || inputs[2 * i + 1].shape() != b0.shape())
+            throw Error("Ternary MatMul group: node " + std::to_string(i) + " has A=" +
+                        shape_str(inputs[2 * i].shape()) + ", B=" + shape_str(inputs[2 * i + 1].shape()) +
+                        ", the group's shape is A=" + shape_str(a0.shape()) + ", B=" + shape_str(b0.shape()));
+    std::vector<Tensor> results;
+    if (m == 0 || n == 0 || k == 0) {
+        for (size_t i = 0; i < count; ++i)
+            results.push_back(Tensor::from_data(std::vector<float>(m * n, 0.0f), {m, n}, DataType::F32,
+                                                TensorLayout::RowMajor));
+        return results;
+    }
+    rbn_ctx *ctx = device_->ctx();
+    // weights: ternarised and tiled once per distinct matrix, as in execute(); cached ones are
+    // pinned for the duration of the call, the others are freed at its end
+    struct Held {
+        rbn_ctx *c;
+        std::vector<void *> owned;
+        std::set<uint64_t> *pins;
+        ~Held() {
+            for (void *p : owned) rbn_free(c, p);
+            pins->clear();
+        }
+    } held{ctx, {}, &pinned_};
+    std::vector<CachedWeights> w(count);
+    for (size_t i = 0; i < count; ++i) {
+        const Tensor &b = inputs[2 * i + 1];
+        const std::vector<float> &bv = b.to_vec();
+        const uint64_t key = cache_weights_ ? hash_floats(bv, b.shape()) : 0;
+        const uint64_t chk = cache_weights_ ? check_bytes(bv.data(), bv.size() * 4) : 0;
+        bool owned = false;
+        w[i] = tiled_weights(key, chk, bv.size() * 4, k, n, nullptr, bv.data(), 1.0f, &owned);
+        if (owned)
+            held.owned.push_back(w[i].d_tiled);
+        else
+            pinned_.insert(key);
+    }
+    // activations: nodes that share their input (q/k/v, gate/up) are quantised once
+    struct Acts {
+        std::unique_ptr<DBuf> q, s, r;
+    };
+    std::vector<Acts> acts;
+    std::vector<size_t> acts_of(count), first_with(0);
+    for (size_t i = 0; i < count; ++i) {
+        const std::vector<float> &av = inputs[2 * i].to_vec();
+        size_t j = 0;
+        for (; j < first_with.size(); ++j) {
+            const std::vector<float> &other = inputs[2 * first_with[j]].to_vec();
+            if (&other == &av || std::memcmp(other.data(), av.data(), av.size() * 4) == 0) break;
+        }
+        acts_of[i] = j;
+        if (j < first_with.size()) continue;
+        first_with.push_back(i);
+        DBuf d_a(ctx, m * k * 4);
+        Acts x;
+        x.q.reset(new DBuf(ctx, m * rbn_act_pitch(k)));
+        x.s.reset(new DBuf(ctx, m * 4));
+        x.r.reset(new DBuf(ctx, m * 4));
+        check(rbn_h2d(ctx, d_a.p, av.data(), m * k * 4), "rbn_h2d");
+        if (act_mode_ == ActivationMode::Ternary)
+            check(rbn_act_quant_ternary(ctx, (const float *)d_a.p, m, k, sum_mode_, (int8_t *)x.q->p,
+                                        (float *)x.s->p, (int32_t *)x.r->p, nullptr, nullptr),
+                  "rbn_act_quant_ternary");
+        else
+            check(rbn_act_quant_i8(ctx, (const float *)d_a.p, m, k, (int8_t *)x.q->p, (float *)x.s->p,
+                                   (int32_t *)x.r->p),
+                  "rbn_act_quant_i8");
+        acts.push_back(std::move(x));
+    }
+    // one output slab, each node's [m,n] block at a 16-byte aligned offset
+    const size_t stride = (m * n * 4 + 15) / 16 * 16;
+    DBuf d_o(ctx, stride * count);
+    const bool decode = m <= RBN_GEMV_MAX_M && rbn_matmul_kernel_choice(m, k, n) == RBN_KERNEL_GEMV;
+    int issued = 0;
+    if (decode) {
+        for (size_t lo = 0; lo < count; lo += RBN_GEMV_GROUP_MAX) {
+            const size_t cnt = std::min<size_t>(RBN_GEMV_GROUP_MAX, count - lo);
+            std::vector<rbn_gemv_problem> problems(cnt);
+            for (size_t i = 0; i < cnt; ++i) {
+                const Acts &x = acts[acts_of[lo + i]];
+                problems[i].d_q = (const int8_t *)x.q->p;
+                problems[i].d_act_scale = (const float *)x.s->p;
+                problems[i].d_rowsum = (const int32_t *)x.r->p;
+                problems[i].d_tiled = (const uint32_t *)w[lo + i].d_tiled;
+                problems[i].w_scale = w[lo + i].scale;
+                problems[i].d_acc = nullptr;
+                problems[i].d_out = (float *)((char *)d_o.p + (lo + i) * stride);
+            }
+            check(rbn_gemv_t2_i8_grouped(ctx, problems.data(), cnt, m, k, n), "rbn_gemv_t2_i8_grouped");
+            ++issued;
+        }
+    } else {
+        for (size_t i = 0; i < count; ++i) {
+            const Acts &x = acts[acts_of[i]];
+            check(rbn_matmul_t2_i8(ctx, (const int8_t *)x.q->p, (const float *)x.s->p, (const int32_t *)x.r->p,
+                                   (const uint32_t *)w[i].d_tiled, w[i].scale, m, k, n, nullptr,
+                                   (float *)((char *)d_o.p + i * stride)),
+                  "rbn_matmul_t2_i8");
+            ++issued;
+        }
+    }
+    std::vector<uint8_t> slab(stride * count);
+    check(rbn_d2h(ctx, slab.data(), d_o.p, slab.size()), "rbn_d2h");
+    for (size_t i = 0; i < count; ++i) {
+        std::vector<float> r(m * n);
+        std::memcpy(r.data(), slab.data() + i * stride, m * n * 4);
+        results.push_back(Tensor::from_data(std::move(r), {m, n}, DataType::F32, TensorLayout::RowMajor));
+    }
+    if (launches) *launches = issued;
+    const double us =
+        std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - start).count();
+    for (size_t i = 0; i < count; ++i) update_stats(us / (double)count);  // one execution per node
+    return results;
 }
 
 Tensor BitNetKernel::execute_prepacked(const Tensor &a, const TernaryTensor &w) {

@@ -19,6 +19,7 @@
 
 #include <atomic>
 #include <mutex>
+#include <set>
 #include <unordered_map>
 
 #include "../../../include/ronn_bitnet_hip.h"
@@ -119,6 +120,16 @@ class BitNetKernel : public CompiledKernel {
     // TernaryMatMul with weights that are already ternarised (e.g. loaded from a packed
     // weight file): A [m,k] f32 is quantised as in execute(), B comes from `w` ([k,n]).
     Tensor execute_prepacked(const Tensor &a, const TernaryTensor &w);
+    // Several independent TernaryMatMul nodes of ONE shape in one call: inputs are the pairs
+    // (A_0, B_0, A_1, B_1, ...), every A_i [m,k] and every B_i [k,n]; result i is what
+    // execute({A_i, B_i}) returns, bit for bit.  These are the nodes a graph holds side by side
+    // (the q/k/v or gate/up projections of one token, the same layer of several sequences) and
+    // that ProviderRegistry::compile_subgraph (registry.rs:237-266) would otherwise run one by
+    // one.  In the decode regime (the shapes rbn_matmul_t2_i8 gives to the GEMV) up to
+    // RBN_GEMV_GROUP_MAX of them become ONE launch of rbn_gemv_t2_i8_grouped, which shares the
+    // fixed cost of a launch between them; other shapes run one launch per node.
+    // *launches (optional) receives the number of matmul launches issued.
+    std::vector<Tensor> execute_group(const std::vector<Tensor> &inputs, int *launches = nullptr);
     MemoryUsage get_memory_usage() const override;
     KernelStats get_performance_stats() const override;
 
@@ -155,6 +166,8 @@ class BitNetKernel : public CompiledKernel {
     std::unordered_map<uint64_t, CachedWeights> weight_cache_;
     size_t cache_bytes_ = 0;
     uint64_t use_clock_ = 0;
+    // keys of cached matrices a running execute_group still needs: never evicted
+    std::set<uint64_t> pinned_;
 };
 
 // kernels.rs:339-344.  Explicit dimensions are checked against the inputs exactly as

@@ -261,6 +261,30 @@ int rbp_kernel_execute(rbp_kernel *k, int n_inputs, const float *const *h_data,
     });
 }
 
+int rbp_kernel_execute_group(rbp_kernel *k, int n_pairs, const float *const *h_a,
+                             const float *const *h_b, const uint64_t shape_a[2],
+                             const uint64_t shape_b[2], float *const *h_out,
+                             uint64_t out_capacity_each, int *launches) {
+    return guarded([&] {
+        if (!k || !h_a || !h_b || !shape_a || !shape_b || !h_out) throw Error("null argument");
+        if (n_pairs < 1) throw Error("Ternary MatMul group requires pairs of inputs (A_i, B_i)");
+        auto *bk = dynamic_cast<BitNetKernel *>(k->k.get());
+        if (!bk) throw Error("not a BitNet kernel");
+        std::vector<Tensor> inputs;
+        for (int i = 0; i < n_pairs; ++i) {
+            inputs.push_back(make_tensor(h_a[i], shape_a, 2, 0));
+            inputs.push_back(make_tensor(h_b[i], shape_b, 2, 0));
+        }
+        std::vector<Tensor> results = bk->execute_group(inputs, launches);
+        for (int i = 0; i < n_pairs; ++i) {
+            const Tensor &r = results.at((size_t)i);
+            if (r.numel() > out_capacity_each) throw Error("output buffer too small");
+            if (!h_out[i]) throw Error("null argument");
+            std::copy(r.to_vec().begin(), r.to_vec().end(), h_out[i]);
+        }
+    });
+}
+
 int rbp_kernel_stats(rbp_kernel *k, uint64_t *execution_count, double *average_us, double *min_us,
                      double *max_us) {
     return guarded([&] {

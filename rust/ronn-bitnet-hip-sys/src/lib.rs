@@ -566,6 +566,17 @@ extern "C" {
         out_capacity: u64,
         out_shape: *mut u64,
     ) -> c_int;
+    pub fn rbp_kernel_execute_group(
+        k: *mut rbp_kernel,
+        n_pairs: c_int,
+        h_a: *const *const f32,
+        h_b: *const *const f32,
+        shape_a: *const u64,
+        shape_b: *const u64,
+        h_out: *const *mut f32,
+        out_capacity_each: u64,
+        launches: *mut c_int,
+    ) -> c_int;
 
 }
 

@@ -351,6 +351,38 @@ def test_gemv_grouped_every_problem_is_its_own_gemv(ctx, M, K, N, count):
             assert (d_acc.download(np.int32, M * N).reshape(M, N) == want_acc).all(), j
 
 
+def test_gemv_grouped_at_the_benchmark_shape(ctx):
+    # the benchmark's step: 32 complete GEMVs of M=1, K=4096, N=11008 in one launch, each with its own
+    # activations and outputs (four distinct weight matrices, eight problems each), every output
+    # against the oracle's integers and epilogue
+    M, K, N, count = 1, 4096, 11008, 32
+    say("gemv grouped", M, K, N, count)
+    mats = []
+    for j in range(4):
+        w = synth_normal(0x5EED1091 + j, 0.02, (K, N))
+        d_p, w_scale, _, _ = ctx.quantize_ternary(ctx.to_device(w), w.size)
+        t, vals = oracle_weights(w)
+        assert bits(w_scale) == bits(t.scale)
+        mats.append((ctx.tile_weights(d_p, K, N), w_scale, t, vals))
+        del w
+    problems, wants = [], []
+    for j in range(count):
+        d_t, w_scale, t, vals = mats[j % 4]
+        x = synth_normal(0x5EED0091 + j, 1.0 + 0.1 * j, (M, K))
+        acts = ctx.act_quant_i8(ctx.to_device(x), M, K)
+        q, s, _ = O.act_quant_i8(x)
+        acc = exact_int_matmul(q, vals)
+        wants.append((acc, epilogue(acc, s, t.scale)))
+        d_out, d_acc = ctx.alloc(4 * M * N), ctx.alloc(4 * M * N)
+        ctx.lib.rbn_fill_u8(ctx.handle, d_out.ptr, 0xFF, 4 * M * N)
+        problems.append((acts, d_t, w_scale, d_out, d_acc))
+    ctx.gemv_grouped(ctx.gemv_problems(problems), M, K, N)
+    ctx.sync()
+    for j, ((acts, d_t, w_scale, d_out, d_acc), (want_acc, want_out)) in enumerate(zip(problems, wants)):
+        assert same_bits(d_out.download(np.float32, M * N).reshape(M, N), want_out), j
+        assert (d_acc.download(np.int32, M * N).reshape(M, N) == want_acc).all(), j
+
+
 def test_gemv_grouped_refused_arguments(ctx):
     d = ctx.alloc(4096)
     probs = ctx.gemv_problems([((d, d, d), d, 1.0, d, None)] * 33)

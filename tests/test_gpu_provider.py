@@ -195,6 +195,74 @@ def test_weight_cache_evicts_least_recently_used():
     assert run(1).allocation_count == 4                      # was evicted: rebuilt
 
 
+def _pairs(a_list, b_list):
+    out = []
+    for a, b in zip(a_list, b_list):
+        out += [Tensor.from_data(a, list(a.shape)), Tensor.from_data(b, list(b.shape))]
+    return out
+
+
+@pytest.mark.parametrize("m,k,n,count,shared_a", [(1, 512, 384, 3, True), (1, 2048, 1000, 2, True),
+                                                  (2, 300, 77, 5, False), (1, 256, 128, 40, False),
+                                                  (8, 256, 192, 2, False), (48, 128, 64, 3, True)])
+def test_execute_group_is_every_node_on_its_own(provider, m, k, n, count, shared_a):
+    # independent MatMul nodes of one shape (q/k/v share their input, other groups do not): each
+    # result against the reference algorithm and against an execute() of its own; in the decode
+    # regime the whole group is one launch (two beyond 32 nodes), other shapes launch per node
+    kernel = provider.compile_subgraph(matmul_subgraph())
+    a0 = synth_normal(900 + m, 1.0, (m, k))
+    a_list = [a0 if shared_a else synth_normal(910 + i, 1.0 + 0.1 * i, (m, k)) for i in range(count)]
+    b_list = [synth_normal(950 + i + n, 0.02, (k, n)) for i in range(count)]
+    outs = kernel.execute_group(_pairs(a_list, b_list))
+    decode = m <= 2
+    assert kernel.last_group_launches == ((count + 31) // 32 if decode else count)
+    assert len(outs) == count
+    for i, (a, b, got) in enumerate(zip(a_list, b_list, outs)):
+        assert got.shape() == [m, n]
+        assert same_bits(got.numpy(), O.execute_ternary(a, b)[0]), i
+        if i < 4:
+            single = kernel.execute([Tensor.from_data(a, [m, k]), Tensor.from_data(b, [k, n])])[0]
+            assert same_bits(got.numpy(), single.numpy()), i
+    assert kernel.get_performance_stats().execution_count == count + min(count, 4)
+
+
+def test_execute_group_int8_activations_and_a_cache_smaller_than_the_group():
+    # room for one 256 x 128 matrix only: the group's other matrices live for the call and are
+    # freed afterwards, the cached one is not evicted under the group's feet
+    p = create_bitnet_provider_with_config(BitNetProviderConfig(activation="int8", max_cache_size=256 * 128 // 4))
+    kernel = p.compile_subgraph(matmul_subgraph())
+    a_list = [synth_normal(1000 + i, 1.0, (1, 256)) for i in range(4)]
+    b_list = [synth_normal(1100 + i, 0.02, (256, 128)) for i in range(4)]
+    for _ in range(2):
+        outs = kernel.execute_group(_pairs(a_list, b_list))
+        assert kernel.last_group_launches == 1
+        for i, (a, b, got) in enumerate(zip(a_list, b_list, outs)):
+            q, sc, _ = O.act_quant_i8(a)
+            want, _ = O.matmul_i8_ternary(q, sc, O.quantize_ternary(b))
+            assert same_bits(got.numpy(), want), i
+    assert kernel.get_memory_usage().current_bytes == 256 * 128 // 4
+
+
+def test_execute_group_input_errors(provider):
+    kernel = provider.compile_subgraph(matmul_subgraph())
+    a = Tensor.from_data(np.ones((1, 64), np.float32), [1, 64])
+    b = Tensor.from_data(np.ones((64, 32), np.float32), [64, 32])
+    with pytest.raises(Error, match="requires pairs of inputs"):
+        kernel.execute_group([a, b, a])
+    with pytest.raises(Error, match="requires pairs of inputs"):
+        kernel.execute_group([])
+    with pytest.raises(Error, match="node 1 has"):
+        kernel.execute_group([a, b, a, Tensor.from_data(np.ones((64, 16), np.float32), [64, 16])])
+    with pytest.raises(Error, match="Matrix dimension mismatch"):
+        kernel.execute_group([b, b])
+    with pytest.raises(Error, match="requires FP32 input tensors"):
+        kernel.execute_group([a, Tensor.from_data(np.ones((64, 32), np.float32), [64, 32], DataType.F16)])
+    sized = provider.create_ternary_matmul_kernel(1, 32, 64)
+    assert len(sized.execute_group([a, b, a, b])) == 2
+    with pytest.raises(Error, match="Matrix dimension mismatch"):
+        provider.create_ternary_matmul_kernel(2, 32, 64).execute_group([a, b])
+
+
 def test_int8_activation_mode():
     p = create_bitnet_provider_with_config(BitNetProviderConfig(activation="int8"))
     kernel = p.compile_subgraph(matmul_subgraph())

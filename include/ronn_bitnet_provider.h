@@ -69,6 +69,11 @@ int rbp_allocate(rbp_provider *p, const uint64_t *shape, int ndim, int dtype, vo
                  uint64_t *size, uint64_t *alignment);
 int rbp_deallocate(rbp_provider *p, void *d_ptr, uint64_t size, uint64_t alignment);
 int rbp_memory_info(rbp_provider *p, uint64_t *total, uint64_t *allocated, uint64_t *peak);
+/* get_memory_stats (provider.rs:121-123) -> BitNetMemoryStats (allocator.rs:157-205); any
+ * out-pointer may be NULL. */
+int rbp_provider_memory_stats(rbp_provider *p, uint64_t *binary_tensor_count,
+                              uint64_t *ternary_tensor_count, uint64_t *memory_saved_bytes,
+                              float *average_compression_ratio);
 
 /* create_ternary_matmul_kernel(m, n, k) (kernels.rs:339-344) on the provider's device. */
 int rbp_create_ternary_matmul_kernel(rbp_provider *p, uint64_t m, uint64_t n, uint64_t k,

@@ -222,6 +222,7 @@ PROVIDER_SIGNATURES = {
     "rbp_allocate": (C.c_int, [_vp, _u64p, C.c_int, C.c_int, C.POINTER(_vp), _u64p, _u64p]),
     "rbp_deallocate": (C.c_int, [_vp, _vp, _u64, _u64]),
     "rbp_memory_info": (C.c_int, [_vp, _u64p, _u64p, _u64p]),
+    "rbp_provider_memory_stats": (C.c_int, [_vp, _u64p, _u64p, _u64p, _f32p]),
     "rbp_create_ternary_matmul_kernel": (C.c_int, [_vp, _u64, _u64, _u64, C.POINTER(_vp)]),
     "rbp_kernel_destroy": (C.c_int, [_vp]),
     "rbp_kernel_execute": (C.c_int, [_vp, C.c_int, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(C.c_int),
@@ -480,6 +481,12 @@ class BitNetExecutionProvider:
     @property
     def config(self) -> BitNetProviderConfig:
         return self.get_config()
+
+    def get_memory_stats(self) -> dict:                              # provider.rs:121-123
+        b, t, saved, ratio = C.c_uint64(), C.c_uint64(), C.c_uint64(), C.c_float()
+        _check(_api().rbp_provider_memory_stats(self._h, C.byref(b), C.byref(t), C.byref(saved), C.byref(ratio)))
+        return {"binary_tensor_count": b.value, "ternary_tensor_count": t.value,
+                "memory_saved_bytes": saved.value, "average_compression_ratio": ratio.value}
 
     def supports_operation(self, op_type: str) -> bool:
         return bool(_api().rbp_provider_supports(self._h, op_type.encode()))

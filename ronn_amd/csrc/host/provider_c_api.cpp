@@ -217,6 +217,19 @@ int rbp_deallocate(rbp_provider *p, void *d_ptr, uint64_t size, uint64_t alignme
     });
 }
 
+int rbp_provider_memory_stats(rbp_provider *p, uint64_t *binary_tensor_count,
+                              uint64_t *ternary_tensor_count, uint64_t *memory_saved_bytes,
+                              float *average_compression_ratio) {
+    return guarded([&] {
+        if (!p) throw Error("provider is NULL");
+        const BitNetMemoryStats &s = p->p->get_memory_stats();
+        if (binary_tensor_count) *binary_tensor_count = s.binary_tensor_count;
+        if (ternary_tensor_count) *ternary_tensor_count = s.ternary_tensor_count;
+        if (memory_saved_bytes) *memory_saved_bytes = s.memory_saved_bytes;
+        if (average_compression_ratio) *average_compression_ratio = s.average_compression_ratio;
+    });
+}
+
 int rbp_memory_info(rbp_provider *p, uint64_t *total, uint64_t *allocated, uint64_t *peak) {
     return guarded([&] {
         if (!p) throw Error("provider is NULL");

@@ -70,10 +70,6 @@ pub const RBN_KERNEL_MFMA: c_int = 2;
 pub const RBN_FLAG_HISTORY_OVERFLOW: u32 = 1;
 pub const RBN_STATIC_SCRATCH_TILES: usize = 1024;
 pub const RBN_STATIC_SCRATCH_BYTES: usize = RBN_STATIC_SCRATCH_TILES * 4096 + 128 * 4;
-// rbn_probe_operands
-pub const RBN_PROBE_CONSTANT: c_int = 0;
-pub const RBN_PROBE_I8_TERNARY: c_int = 1;
-pub const RBN_PROBE_I8_I8: c_int = 2;
 
 // DataType codes of rbn_tensor_bytes / rbp_* (declaration order of ronn_core::DataType,
 // crates/ronn-core/src/types.rs:39-60)
@@ -432,14 +428,6 @@ extern "C" {
         d_out: *mut f32,
         n: u64,
     ) -> c_int;
-    pub fn rbn_probe_mfma_i8(ctx: *mut rbn_ctx, operand_kind: c_int, h_tops: *mut f64) -> c_int;
-    pub fn rbn_probe_empty_launch(ctx: *mut rbn_ctx) -> c_int;
-    pub fn rbn_probe_stream_read(
-        ctx: *mut rbn_ctx,
-        d_src: *const c_void,
-        bytes: u64,
-        nontemporal: c_int,
-    ) -> c_int;
     pub fn rbn_synth_normal_f32(seed: u64, sigma: f64, first: u64, count: u64, h_out: *mut f32);
 // ---- include/ronn_bitnet_provider.h ----
     pub fn rbp_last_error() -> *const c_char;
@@ -486,6 +474,13 @@ extern "C" {
         total: *mut u64,
         allocated: *mut u64,
         peak: *mut u64,
+    ) -> c_int;
+    pub fn rbp_provider_memory_stats(
+        p: *mut rbp_provider,
+        binary_tensor_count: *mut u64,
+        ternary_tensor_count: *mut u64,
+        memory_saved_bytes: *mut u64,
+        average_compression_ratio: *mut f32,
     ) -> c_int;
     pub fn rbp_create_ternary_matmul_kernel(
         p: *mut rbp_provider,

@@ -1,268 +1,194 @@
 //! `CompiledKernel` for the TernaryMatMul operation on the GPU.
 //!
 //! Stands in for `BitNetKernel` with `BitNetOperation::TernaryMatMul`
-//! (crates/ronn-providers/src/bitnet/kernels.rs:36-47, :134-178, :254-328).
+//! (crates/ronn-providers/src/bitnet/kernels.rs:36-47, :134-178, :254-328).  The kernel object
+//! itself lives behind the C ABI (`rbp_kernel`): weight cache (ternarise once, two digests,
+//! least-recently-used eviction), activation quantisation, kernel choice and statistics are the
+//! library's, so this file only moves tensors across the boundary.
 
-use std::collections::hash_map::DefaultHasher;
-use std::collections::HashMap;
-use std::hash::{Hash, Hasher};
-use std::os::raw::{c_int, c_void};
+use std::os::raw::c_int;
 use std::ptr::null_mut;
-use std::sync::{Arc, Mutex};
-use std::time::Instant;
 
 use anyhow::{anyhow, Result};
 use ronn_bitnet_hip_sys as sys;
 use ronn_core::{CompiledKernel, DataType, KernelStats, MemoryUsage, Tensor, TensorLayout};
 
-use crate::provider::ActivationMode;
-
-fn check(rc: c_int) -> Result<()> {
-    sys::check(rc).map_err(|m| anyhow!(m))
+/// The library's message for the calling thread's last provider-level failure; for errors the
+/// reference also raises it is the reference's text.
+pub(crate) fn check(rc: c_int) -> Result<()> {
+    sys::check_provider(rc).map_err(|m| anyhow!(m))
 }
 
-/// Owns one `rbn_ctx` (one GPU, one stream).  The C side locks the context around every call,
-/// which is what makes sharing it between threads sound.
-pub struct HipContext {
-    raw: *mut sys::rbn_ctx,
-}
-
-// SAFETY: every entry point that takes the context serialises its callers with the context's
-// own lock and makes the context's device current for the calling thread.
-unsafe impl Send for HipContext {}
-unsafe impl Sync for HipContext {}
-
-impl HipContext {
-    pub fn new(device: i32) -> Result<Arc<Self>> {
-        let mut raw = null_mut();
-        // SAFETY: `raw` is a valid out-pointer.
-        check(unsafe { sys::rbn_ctx_create(device as c_int, &mut raw) })?;
-        Ok(Arc::new(Self { raw }))
-    }
-
-    pub fn raw(&self) -> *mut sys::rbn_ctx {
-        self.raw
-    }
-
-    /// Device allocation that frees itself.
-    pub fn alloc(self: &Arc<Self>, bytes: usize) -> Result<DeviceBuffer> {
-        let mut p: *mut c_void = null_mut();
-        // SAFETY: `p` is a valid out-pointer.
-        check(unsafe { sys::rbn_malloc(self.raw, bytes, &mut p) })?;
-        Ok(DeviceBuffer { ctx: Arc::clone(self), ptr: p, bytes })
-    }
-
-    pub fn upload(self: &Arc<Self>, data: &[f32]) -> Result<DeviceBuffer> {
-        let buf = self.alloc(std::mem::size_of_val(data).max(4))?;
-        // SAFETY: `buf` has at least `data.len() * 4` bytes.
-        check(unsafe { sys::rbn_h2d(self.raw, buf.ptr, data.as_ptr().cast(), std::mem::size_of_val(data)) })?;
-        Ok(buf)
+fn dtype_code(dtype: DataType) -> c_int {
+    match dtype {
+        DataType::F32 => sys::RBN_DT_F32,
+        DataType::F16 => sys::RBN_DT_F16,
+        DataType::BF16 => sys::RBN_DT_BF16,
+        DataType::I8 => sys::RBN_DT_I8,
+        DataType::I32 => sys::RBN_DT_I32,
+        DataType::I64 => sys::RBN_DT_I64,
+        DataType::U8 => sys::RBN_DT_U8,
+        DataType::U32 => sys::RBN_DT_U32,
+        DataType::Bool => sys::RBN_DT_BOOL,
+        DataType::F64 => sys::RBN_DT_F64,
     }
 }
 
-impl Drop for HipContext {
-    fn drop(&mut self) {
-        // SAFETY: created by rbn_ctx_create and not used after this.
-        unsafe { sys::rbn_ctx_destroy(self.raw) };
+pub(crate) fn dtype_to_code(dtype: DataType) -> c_int {
+    dtype_code(dtype)
+}
+
+/// One compiled BitNet kernel on the GPU.
+pub struct HipKernel {
+    raw: *mut sys::rbp_kernel,
+}
+
+// SAFETY: the object behind `raw` takes its own lock for the whole of every call
+// (`CompiledKernel` is `Send + Sync`, types.rs:153: `execute(&self)` may run on many threads).
+unsafe impl Send for HipKernel {}
+unsafe impl Sync for HipKernel {}
+
+impl HipKernel {
+    /// Takes ownership of a kernel created by `rbp_provider_compile_subgraph` or
+    /// `rbp_create_ternary_matmul_kernel`.
+    pub(crate) fn from_raw(raw: *mut sys::rbp_kernel) -> Self {
+        Self { raw }
     }
-}
 
-pub struct DeviceBuffer {
-    ctx: Arc<HipContext>,
-    ptr: *mut c_void,
-    bytes: usize,
-}
-
-unsafe impl Send for DeviceBuffer {}
-unsafe impl Sync for DeviceBuffer {}
-
-impl DeviceBuffer {
-    pub fn ptr<T>(&self) -> *mut T {
-        self.ptr.cast()
-    }
-    pub fn bytes(&self) -> usize {
-        self.bytes
-    }
-}
-
-impl Drop for DeviceBuffer {
-    fn drop(&mut self) {
-        // SAFETY: allocated by rbn_malloc on this context; rbn_free waits for the stream first.
-        unsafe { sys::rbn_free(self.ctx.raw, self.ptr) };
-    }
-}
-
-/// A weight matrix ternarised once (`quantize_ternary`, quantization.rs:67-109) and laid out for
-/// the matmul kernels.
-struct TiledWeights {
-    tiled: DeviceBuffer,
-    scale: f32,
-    k: u64,
-    n: u64,
-    /// Second, independent digest of the f32 data: a hit on the first key alone is not trusted.
-    check: u64,
-}
-
-/// TernaryMatMul on the GPU.
-pub struct HipTernaryMatMul {
-    ctx: Arc<HipContext>,
-    /// Ternarised weights by content key; the reference re-ternarises input 1 on every call
-    /// (kernels.rs:278), here that happens once per distinct matrix.
-    weights: Mutex<HashMap<u64, Arc<TiledWeights>>>,
-    stats: Mutex<KernelStats>,
-    memory: Mutex<MemoryUsage>,
-    sum_mode: c_int,
-    activation: ActivationMode,
-    max_cache_bytes: usize,
-}
-
-impl HipTernaryMatMul {
-    pub fn new(ctx: Arc<HipContext>, strict_reference_sum: bool, activation: ActivationMode,
-               max_cache_bytes: usize) -> Self {
-        Self {
-            ctx,
-            weights: Mutex::new(HashMap::new()),
-            stats: Mutex::new(KernelStats {
-                execution_count: 0,
-                average_time_us: 0.0,
-                min_time_us: 0.0,
-                max_time_us: 0.0,
-            }),
-            memory: Mutex::new(MemoryUsage { peak_bytes: 0, current_bytes: 0, allocation_count: 0 }),
-            sum_mode: if strict_reference_sum { sys::RBN_SUM_STRICT_SEQ } else { sys::RBN_SUM_TREE },
-            activation,
-            max_cache_bytes,
+    /// Several independent TernaryMatMul nodes of one shape in one call: `pairs[i] = (A_i, B_i)`,
+    /// every `A_i` `[m,k]`, every `B_i` `[k,n]`.  Result `i` is what `execute(&[A_i, B_i])`
+    /// returns, bit for bit.  A graph holds such nodes side by side (the q/k/v or gate/up
+    /// projections of one token; `ProviderRegistry::compile_subgraph`, registry.rs:237-266,
+    /// compiles them one by one); in the decode regime the library runs up to 32 of them as one
+    /// GPU launch, which is what brings a single-token matmul from a third of the memory
+    /// bandwidth towards all of it.  Returns the results and the number of launches issued.
+    pub fn execute_group(&self, pairs: &[(&Tensor, &Tensor)]) -> Result<(Vec<Tensor>, usize)> {
+        if pairs.is_empty() {
+            return Err(anyhow!("Ternary MatMul group requires pairs of inputs (A_i, B_i)"));
         }
-    }
-
-    fn digests(data: &[f32]) -> (u64, u64) {
-        let mut h1 = DefaultHasher::new();
-        let mut h2: u64 = 0xcbf2_9ce4_8422_2325; // FNV-1a over the bit patterns
-        data.len().hash(&mut h1);
-        for v in data {
-            let b = v.to_bits();
-            b.hash(&mut h1);
-            h2 = (h2 ^ u64::from(b)).wrapping_mul(0x0000_0100_0000_01b3);
-        }
-        (h1.finish(), h2)
-    }
-
-    /// quantize_ternary + tiling of input 1, cached.
-    fn tiled_weights(&self, b: &Tensor, k: u64, n: u64) -> Result<Arc<TiledWeights>> {
-        let data = b.to_vec()?; // tensor.rs:217, row-major
-        let (key, check_digest) = Self::digests(&data);
-        if let Some(w) = self.weights.lock().unwrap().get(&key) {
-            if w.k == k && w.n == n && w.check == check_digest {
-                return Ok(Arc::clone(w));
-            }
-        }
-        let ctx = &self.ctx;
-        let d_w = ctx.upload(&data)?;
-        // SAFETY: sizes come from the library's own size functions; all buffers are live until
-        // the synchronous calls below have returned.
-        let w = unsafe {
-            let d_packed = ctx.alloc(sys::rbn_packed_capacity(k * n))?;
-            let (mut scale, mut threshold, mut survivors) = (0f32, 0f32, 0u64);
-            check(sys::rbn_quantize_ternary(ctx.raw(), d_w.ptr(), k * n, self.sum_mode, d_packed.ptr(),
-                                            &mut scale, &mut threshold, &mut survivors))?;
-            let tiled = ctx.alloc(sys::rbn_tiled_bytes(k, n))?;
-            check(sys::rbn_tile_weights(ctx.raw(), d_packed.ptr(), k, n, tiled.ptr()))?;
-            check(sys::rbn_sync(ctx.raw()))?;
-            Arc::new(TiledWeights { tiled, scale, k, n, check: check_digest })
-        };
-        let mut cache = self.weights.lock().unwrap();
-        let mut mem = self.memory.lock().unwrap();
-        // no room: drop the cached matrices (they are rebuilt on demand) rather than grow
-        if mem.current_bytes + w.tiled.bytes() > self.max_cache_bytes {
-            cache.clear();
-            mem.current_bytes = 0;
-        }
-        mem.current_bytes += w.tiled.bytes();
-        mem.peak_bytes = mem.peak_bytes.max(mem.current_bytes);
-        mem.allocation_count += 1;
-        cache.insert(key, Arc::clone(&w));
-        Ok(w)
-    }
-
-    /// kernels.rs:235-251.
-    fn update_stats(&self, execution_time_us: f64) {
-        let mut s = self.stats.lock().unwrap();
-        s.execution_count += 1;
-        if s.execution_count == 1 {
-            s.min_time_us = execution_time_us;
-            s.max_time_us = execution_time_us;
-            s.average_time_us = execution_time_us;
-        } else {
-            s.min_time_us = s.min_time_us.min(execution_time_us);
-            s.max_time_us = s.max_time_us.max(execution_time_us);
-            let n = s.execution_count as f64;
-            s.average_time_us = ((n - 1.0) * s.average_time_us + execution_time_us) / n;
-        }
-    }
-}
-
-impl CompiledKernel for HipTernaryMatMul {
-    fn execute(&self, inputs: &[Tensor]) -> Result<Vec<Tensor>> {
-        let start_time = Instant::now();
-        if inputs.len() != 2 {
-            return Err(anyhow!("Ternary MatMul requires exactly 2 inputs")); // kernels.rs:273
-        }
-        for t in inputs {
-            if t.dtype() != DataType::F32 {
+        for (a, b) in pairs {
+            if a.dtype() != DataType::F32 || b.dtype() != DataType::F32 {
                 // quantization.rs:68-72
                 return Err(anyhow!("BitNet quantization requires FP32 input tensors"));
             }
         }
-        let (a, b) = (&inputs[0], &inputs[1]);
-        let (sa, sb) = (a.shape(), b.shape());
-        // kernels.rs:142-152; m, n, k come from the inputs instead of the constants 64, 64, 64
-        if sa.len() != 2 || sb.len() != 2 || sa[1] != sb[0] {
-            return Err(anyhow!(
-                "Matrix dimension mismatch: A={:?}, B={:?}, expected A=[m,k], B=[k,n]",
-                sa, sb
-            ));
-        }
-        let (m, k, n) = (sa[0] as u64, sa[1] as u64, sb[1] as u64);
-        if m == 0 || k == 0 || n == 0 {
+        let (sa, sb) = (pairs[0].0.shape(), pairs[0].1.shape());
+        if sa.len() != 2 || sb.len() != 2 {
             return Err(anyhow!("Matrix dimension mismatch: A={:?}, B={:?}, expected A=[m,k], B=[k,n]", sa, sb));
         }
-        let w = self.tiled_weights(b, k, n)?;
-        let ctx = &self.ctx;
-        let av = a.to_vec()?;
-        let d_a = ctx.upload(&av)?;
-        let mut out = vec![0f32; (m * n) as usize];
-        // SAFETY: buffer sizes follow the header (m * rbn_act_pitch(k) int8, m f32, m int32,
-        // m * n f32); rbn_d2h synchronises the stream before `out` is read.
-        unsafe {
-            let d_q = ctx.alloc(m as usize * sys::rbn_act_pitch(k))?;
-            let d_scale = ctx.alloc(4 * m as usize)?;
-            let d_rowsum = ctx.alloc(4 * m as usize)?;
-            match self.activation {
-                // per-token absmax int8 (no counterpart in the reference)
-                ActivationMode::Int8PerToken => check(sys::rbn_act_quant_i8(
-                    ctx.raw(), d_a.ptr(), m, k, d_q.ptr(), d_scale.ptr(), d_rowsum.ptr()))?,
-                // the reference's own choice: quantize_ternary over the whole tensor (kernels.rs:277)
-                ActivationMode::TernaryPerTensor => check(sys::rbn_act_quant_ternary(
-                    ctx.raw(), d_a.ptr(), m, k, self.sum_mode, d_q.ptr(), d_scale.ptr(), d_rowsum.ptr(),
-                    null_mut(), null_mut()))?,
+        // the C entry point takes one shape for the whole group
+        for (i, (a, b)) in pairs.iter().enumerate().skip(1) {
+            if a.shape() != sa || b.shape() != sb {
+                return Err(anyhow!(
+                    "Ternary MatMul group: node {} has A={:?}, B={:?}, the group's shape is A={:?}, B={:?}",
+                    i, a.shape(), b.shape(), sa, sb
+                ));
             }
-            let d_out = ctx.alloc(4 * (m * n) as usize)?;
-            // kernels.rs:134-178 with the epilogue of :168
-            check(sys::rbn_matmul_t2_i8(ctx.raw(), d_q.ptr(), d_scale.ptr(), d_rowsum.ptr(), w.tiled.ptr(),
-                                        w.scale, m, k, n, null_mut(), d_out.ptr()))?;
-            check(sys::rbn_d2h(ctx.raw(), out.as_mut_ptr().cast(), d_out.ptr::<c_void>() as *const c_void,
-                               out.len() * 4))?;
         }
-        let result = Tensor::from_data(out, vec![m as usize, n as usize], DataType::F32, TensorLayout::RowMajor)?;
-        self.update_stats(start_time.elapsed().as_micros() as f64);
-        Ok(vec![result])
+        let a_data: Vec<Vec<f32>> = pairs.iter().map(|(a, _)| a.to_vec()).collect::<Result<_>>()?;
+        let b_data: Vec<Vec<f32>> = pairs.iter().map(|(_, b)| b.to_vec()).collect::<Result<_>>()?;
+        let (m, n) = (sa[0], sb[1]);
+        let mut outs: Vec<Vec<f32>> = pairs.iter().map(|_| vec![0f32; (m * n).max(1)]).collect();
+        let pa: Vec<*const f32> = a_data.iter().map(|v| v.as_ptr()).collect();
+        let pb: Vec<*const f32> = b_data.iter().map(|v| v.as_ptr()).collect();
+        let po: Vec<*mut f32> = outs.iter_mut().map(|v| v.as_mut_ptr()).collect();
+        let shape_a = [sa[0] as u64, sa[1] as u64];
+        let shape_b = [sb[0] as u64, sb[1] as u64];
+        let mut launches: c_int = 0;
+        // SAFETY: every pointer array has `pairs.len()` live entries; each input holds the number
+        // of elements its shape says (Tensor::to_vec); each output has `out_capacity_each` elements.
+        check(unsafe {
+            sys::rbp_kernel_execute_group(
+                self.raw,
+                pairs.len() as c_int,
+                pa.as_ptr(),
+                pb.as_ptr(),
+                shape_a.as_ptr(),
+                shape_b.as_ptr(),
+                po.as_ptr(),
+                (m * n).max(1) as u64,
+                &mut launches,
+            )
+        })?;
+        let mut results = Vec::with_capacity(outs.len());
+        for mut o in outs {
+            o.truncate(m * n);
+            results.push(Tensor::from_data(o, vec![m, n], DataType::F32, TensorLayout::RowMajor)?);
+        }
+        Ok((results, launches as usize))
+    }
+}
+
+impl Drop for HipKernel {
+    fn drop(&mut self) {
+        // SAFETY: created by the library, not used after this.
+        unsafe { sys::rbp_kernel_destroy(self.raw) };
+    }
+}
+
+impl CompiledKernel for HipKernel {
+    /// kernels.rs:254-319.  Input checks, error texts ("Ternary MatMul requires exactly 2
+    /// inputs", "Matrix dimension mismatch: ...", "BitNet quantization requires FP32 input
+    /// tensors") and the arithmetic are the library's; m, n, k come from the inputs.
+    fn execute(&self, inputs: &[Tensor]) -> Result<Vec<Tensor>> {
+        let data: Vec<Vec<f32>> = inputs
+            .iter()
+            .map(|t| if t.dtype() == DataType::F32 { t.to_vec() } else { Ok(Vec::new()) })
+            .collect::<Result<_>>()?;
+        let shapes: Vec<Vec<u64>> = inputs.iter().map(|t| t.shape().iter().map(|&d| d as u64).collect()).collect();
+        let data_p: Vec<*const f32> = data.iter().map(|v| v.as_ptr()).collect();
+        let shape_p: Vec<*const u64> = shapes.iter().map(|v| v.as_ptr()).collect();
+        let ndims: Vec<c_int> = shapes.iter().map(|v| v.len() as c_int).collect();
+        let dtypes: Vec<c_int> = inputs.iter().map(|t| dtype_code(t.dtype())).collect();
+        // [m, n] of a well-formed call; anything else is rejected by the library before it writes
+        let capacity = match (shapes.first(), shapes.get(1)) {
+            (Some(a), Some(b)) if a.len() == 2 && b.len() == 2 => (a[0] * b[1]).max(1) as usize,
+            _ => 1,
+        };
+        let mut out = vec![0f32; capacity];
+        let mut out_shape = [0u64; 2];
+        // SAFETY: the arrays have `inputs.len()` live entries; a non-F32 tensor is refused on its
+        // dtype code before its (empty) data is looked at; `out` has `capacity` elements.
+        check(unsafe {
+            sys::rbp_kernel_execute(
+                self.raw,
+                inputs.len() as c_int,
+                data_p.as_ptr(),
+                shape_p.as_ptr(),
+                ndims.as_ptr(),
+                dtypes.as_ptr(),
+                out.as_mut_ptr(),
+                capacity as u64,
+                out_shape.as_mut_ptr(),
+            )
+        })?;
+        let (m, n) = (out_shape[0] as usize, out_shape[1] as usize);
+        out.truncate(m * n);
+        Ok(vec![Tensor::from_data(out, vec![m, n], DataType::F32, TensorLayout::RowMajor)?])
     }
 
+    /// kernels.rs:321-323; here the bytes of cached, ternarised weights.
     fn get_memory_usage(&self) -> MemoryUsage {
-        self.memory.lock().unwrap().clone()
+        let (mut peak, mut current, mut allocations) = (0u64, 0u64, 0u64);
+        // SAFETY: valid out-pointers.
+        let _ = unsafe { sys::rbp_kernel_memory_usage(self.raw, &mut peak, &mut current, &mut allocations) };
+        MemoryUsage {
+            peak_bytes: peak as usize,
+            current_bytes: current as usize,
+            allocation_count: allocations as usize,
+        }
     }
 
+    /// kernels.rs:325-327; really updated (the reference measures and drops, :313-316).
     fn get_performance_stats(&self) -> KernelStats {
-        self.stats.lock().unwrap().clone()
+        let (mut count, mut avg, mut lo, mut hi) = (0u64, 0f64, 0f64, 0f64);
+        // SAFETY: valid out-pointers.
+        let _ = unsafe { sys::rbp_kernel_stats(self.raw, &mut count, &mut avg, &mut lo, &mut hi) };
+        KernelStats { execution_count: count, average_time_us: avg, min_time_us: lo, max_time_us: hi }
     }
+}
+
+/// Keeps `null_mut` in one place for the callers that create kernels.
+pub(crate) fn null_kernel() -> *mut sys::rbp_kernel {
+    null_mut()
 }

@@ -17,8 +17,8 @@
 pub mod hip_kernel;
 pub mod provider;
 
-pub use hip_kernel::{HipContext, HipTernaryMatMul};
+pub use hip_kernel::HipKernel;
 pub use provider::{
     create_bitnet_provider, create_bitnet_provider_with_config, ActivationMode, BitNetExecutionProvider,
-    BitNetHipAllocator, BitNetProviderConfig, QuantizationMethod,
+    BitNetHipAllocator, BitNetMemoryStats, BitNetProviderConfig, QuantizationMethod,
 };

@@ -1,24 +1,27 @@
 //! `ExecutionProvider` with `ProviderId::BitNet` on an MI355X.
 //!
 //! Stands in for `BitNetExecutionProvider` (crates/ronn-providers/src/bitnet/provider.rs:25-398)
-//! and `BitNetMemoryAllocator` (bitnet/allocator.rs:15-149).
+//! and `BitNetMemoryAllocator` (bitnet/allocator.rs:15-149).  The provider object, its
+//! configuration rules, its supported-operation set, its speed-up table and its error texts live
+//! behind the C ABI (`rbp_provider`), where the GPU tests exercise them; this file converts between
+//! the traits' Rust types and that ABI.
 
 use std::collections::HashSet;
-use std::os::raw::{c_int, c_void};
+use std::ffi::CString;
+use std::os::raw::{c_char, c_int, c_void};
 use std::ptr::null_mut;
-use std::sync::atomic::{AtomicUsize, Ordering};
 use std::sync::Arc;
 
 use anyhow::{anyhow, Result};
 use ronn_bitnet_hip_sys as sys;
 use ronn_core::{
-    CompiledKernel, DataType, ExecutionProvider, GraphNode, MemoryInfo, MemoryType, OperatorSpec,
-    OptimizationLevel, PerformanceProfile, ProviderCapability, ProviderConfig, ProviderId,
-    ResourceRequirements, SubGraph, TensorAllocator, TensorBuffer,
+    CompiledKernel, DataType, ExecutionProvider, MemoryInfo, MemoryType, OperatorSpec, OptimizationLevel,
+    PerformanceProfile, ProviderCapability, ProviderConfig, ProviderId, ResourceRequirements, SubGraph,
+    TensorAllocator, TensorBuffer,
 };
-use tracing::{debug, info, warn};
+use tracing::{debug, info};
 
-use crate::hip_kernel::{HipContext, HipTernaryMatMul};
+use crate::hip_kernel::{check, dtype_to_code, null_kernel, HipKernel};
 
 /// provider.rs of the reference takes this from bitnet/quantization.rs:13-20; same variants.
 #[derive(Debug, Clone, Copy, PartialEq)]
@@ -55,103 +58,132 @@ pub struct BitNetProviderConfig {
     pub device: i32,
 }
 
-impl Default for BitNetProviderConfig {
-    fn default() -> Self {
-        Self {
-            // the reference defaults to Binary (provider.rs:60); only the ternary half exists here
-            quantization_method: QuantizationMethod::Ternary,
-            enable_kernel_caching: true,
-            max_cache_size: 64 * 1024 * 1024,
-            enable_mixed_precision: true,
-            memory_optimization_level: 2,
-            enable_simd: true,
-            activation: ActivationMode::TernaryPerTensor,
-            strict_reference_sum: true,
-            device: 0,
+impl BitNetProviderConfig {
+    fn to_c(&self) -> sys::rbp_config {
+        sys::rbp_config {
+            quantization_method: match self.quantization_method {
+                QuantizationMethod::Binary => 0,
+                QuantizationMethod::Ternary => 1,
+                QuantizationMethod::AsymmetricBinary { .. } => 2,
+            },
+            enable_kernel_caching: self.enable_kernel_caching as c_int,
+            max_cache_size: self.max_cache_size as u64,
+            enable_mixed_precision: self.enable_mixed_precision as c_int,
+            memory_optimization_level: c_int::from(self.memory_optimization_level),
+            enable_simd: self.enable_simd as c_int,
+            activation: (self.activation == ActivationMode::Int8PerToken) as c_int,
+            strict_reference_sum: self.strict_reference_sum as c_int,
+            device: self.device as c_int,
         }
+    }
+
+    fn from_c(c: &sys::rbp_config) -> Self {
+        Self {
+            quantization_method: match c.quantization_method {
+                0 => QuantizationMethod::Binary,
+                2 => QuantizationMethod::AsymmetricBinary { threshold: 0.0 },
+                _ => QuantizationMethod::Ternary,
+            },
+            enable_kernel_caching: c.enable_kernel_caching != 0,
+            max_cache_size: c.max_cache_size as usize,
+            enable_mixed_precision: c.enable_mixed_precision != 0,
+            memory_optimization_level: c.memory_optimization_level as u8,
+            enable_simd: c.enable_simd != 0,
+            activation: if c.activation != 0 { ActivationMode::Int8PerToken } else { ActivationMode::TernaryPerTensor },
+            strict_reference_sum: c.strict_reference_sum != 0,
+            device: c.device as i32,
+        }
+    }
+}
+
+impl Default for BitNetProviderConfig {
+    /// The library's defaults: as provider.rs:57-68, except that the method is Ternary (the
+    /// reference defaults to Binary, :60; only the ternary half exists here).
+    fn default() -> Self {
+        // SAFETY: plain-old-data out-parameter, filled in full.
+        let mut c: sys::rbp_config = unsafe { std::mem::zeroed() };
+        unsafe { sys::rbp_default_config(&mut c) };
+        Self::from_c(&c)
+    }
+}
+
+/// `BitNetMemoryStats` (allocator.rs:157-205) as `get_memory_stats` reports it.
+#[derive(Debug, Clone, Copy, PartialEq)]
+pub struct BitNetMemoryStats {
+    pub binary_tensor_count: usize,
+    pub ternary_tensor_count: usize,
+    pub memory_saved_bytes: usize,
+    pub average_compression_ratio: f32,
+}
+
+/// Owns the library's provider object.
+struct ProviderHandle {
+    raw: *mut sys::rbp_provider,
+}
+
+// SAFETY: the object's const operations are read-only or go through the device context, which
+// takes its own lock for every call; `configure` needs `&mut BitNetExecutionProvider`.
+unsafe impl Send for ProviderHandle {}
+unsafe impl Sync for ProviderHandle {}
+
+impl Drop for ProviderHandle {
+    fn drop(&mut self) {
+        // SAFETY: created by rbp_provider_create and not used after this.
+        unsafe { sys::rbp_provider_destroy(self.raw) };
     }
 }
 
 /// Device-memory `TensorAllocator` with the reference's size and alignment rules
 /// (allocator.rs:39-75): U8 = 2-bit ternary, 4 elements per byte; Bool = 1 bit per element.
 pub struct BitNetHipAllocator {
-    ctx: Arc<HipContext>,
-    allocated_bytes: AtomicUsize,
-    peak_bytes: AtomicUsize,
-    total_bytes: usize,
-}
-
-fn dtype_code(dtype: DataType) -> c_int {
-    match dtype {
-        DataType::F32 => sys::RBN_DT_F32,
-        DataType::F16 => sys::RBN_DT_F16,
-        DataType::BF16 => sys::RBN_DT_BF16,
-        DataType::I8 => sys::RBN_DT_I8,
-        DataType::I32 => sys::RBN_DT_I32,
-        DataType::I64 => sys::RBN_DT_I64,
-        DataType::U8 => sys::RBN_DT_U8,
-        DataType::U32 => sys::RBN_DT_U32,
-        DataType::Bool => sys::RBN_DT_BOOL,
-        DataType::F64 => sys::RBN_DT_F64,
-    }
-}
-
-impl BitNetHipAllocator {
-    pub fn new(ctx: Arc<HipContext>) -> Result<Self> {
-        // SAFETY: plain-old-data out-parameter.
-        let mut info: sys::rbn_device_info = unsafe { std::mem::zeroed() };
-        sys::check(unsafe { sys::rbn_get_device_info(ctx.raw(), &mut info) }).map_err(|m| anyhow!(m))?;
-        Ok(Self {
-            ctx,
-            allocated_bytes: AtomicUsize::new(0),
-            peak_bytes: AtomicUsize::new(0),
-            total_bytes: info.hbm_bytes as usize,
-        })
-    }
+    provider: Arc<ProviderHandle>,
 }
 
 impl TensorAllocator for BitNetHipAllocator {
+    /// allocator.rs:100-128; an unsupported dtype gives the reference's message (:61-64).
     fn allocate(&self, shape: &[usize], dtype: DataType) -> Result<TensorBuffer> {
-        let element_count: usize = shape.iter().product();
-        // SAFETY: pure functions of their arguments.
-        let size = unsafe { sys::rbn_tensor_bytes(element_count as u64, dtype_code(dtype)) };
-        if size < 0 {
-            // allocator.rs:61-64
-            return Err(anyhow!("Unsupported data type for BitNet allocator: {:?}", dtype));
-        }
-        let size = size as usize;
-        let alignment = unsafe { sys::rbn_tensor_alignment(dtype_code(dtype)) };
+        let dims: Vec<u64> = shape.iter().map(|&d| d as u64).collect();
         let mut p: *mut c_void = null_mut();
-        // SAFETY: valid out-pointer; device memory comes back 256-byte aligned.
-        sys::check(unsafe { sys::rbn_malloc(self.ctx.raw(), size, &mut p) })
-            .map_err(|m| anyhow!("Memory allocation failed for {} bytes: {}", size, m))?;
-        let now = self.allocated_bytes.fetch_add(size, Ordering::Relaxed) + size;
-        self.peak_bytes.fetch_max(now, Ordering::Relaxed);
-        Ok(TensorBuffer { ptr: p.cast(), size, alignment, memory_type: MemoryType::DeviceMemory })
+        let (mut size, mut alignment) = (0u64, 0u64);
+        // SAFETY: `dims` has `dims.len()` entries; valid out-pointers.
+        check(unsafe {
+            sys::rbp_allocate(self.provider.raw, dims.as_ptr(), dims.len() as c_int, dtype_to_code(dtype), &mut p,
+                              &mut size, &mut alignment)
+        })?;
+        Ok(TensorBuffer {
+            ptr: p.cast(),
+            size: size as usize,
+            alignment: alignment as usize,
+            memory_type: MemoryType::DeviceMemory,
+        })
     }
 
+    /// allocator.rs:130-140.
     fn deallocate(&self, buffer: TensorBuffer) -> Result<()> {
-        // SAFETY: `buffer.ptr` came from `allocate` above.
-        sys::check(unsafe { sys::rbn_free(self.ctx.raw(), buffer.ptr.cast()) }).map_err(|m| anyhow!(m))?;
-        self.allocated_bytes.fetch_sub(buffer.size, Ordering::Relaxed);
-        Ok(())
+        // SAFETY: `buffer` came from `allocate` above.
+        check(unsafe {
+            sys::rbp_deallocate(self.provider.raw, buffer.ptr.cast(), buffer.size as u64, buffer.alignment as u64)
+        })
     }
 
+    /// allocator.rs:142-148.
     fn get_memory_info(&self) -> MemoryInfo {
-        MemoryInfo {
-            total_bytes: self.total_bytes,
-            allocated_bytes: self.allocated_bytes.load(Ordering::Relaxed),
-            peak_bytes: self.peak_bytes.load(Ordering::Relaxed),
-        }
+        let (mut total, mut allocated, mut peak) = (0u64, 0u64, 0u64);
+        // SAFETY: valid out-pointers.
+        let _ = unsafe { sys::rbp_memory_info(self.provider.raw, &mut total, &mut allocated, &mut peak) };
+        MemoryInfo { total_bytes: total as usize, allocated_bytes: allocated as usize, peak_bytes: peak as usize }
     }
 }
 
+/// The operation names `get_capability` can report (provider.rs:87-99); which of them the
+/// provider supports is the library's answer.
+const OP_NAMES: [&str; 12] =
+    ["MatMul", "Gemm", "Conv", "Add", "Sub", "Mul", "And", "Or", "Xor", "BatchNormalization", "ReLU", "Sigmoid"];
+
 /// BitNet execution provider backed by the gfx950 kernels.
 pub struct BitNetExecutionProvider {
-    config: BitNetProviderConfig,
-    ctx: Arc<HipContext>,
+    handle: Arc<ProviderHandle>,
     allocator: Arc<dyn TensorAllocator>,
-    supported_ops: HashSet<String>,
 }
 
 impl BitNetExecutionProvider {
@@ -159,72 +191,66 @@ impl BitNetExecutionProvider {
         Self::with_config(BitNetProviderConfig::default())
     }
 
-    /// provider.rs:77-114: resources and the supported-operation set.
+    /// provider.rs:77-114.
     pub fn with_config(config: BitNetProviderConfig) -> Result<Self> {
         info!("Creating BitNet execution provider with method: {:?}", config.quantization_method);
-        let ctx = HipContext::new(config.device)?;
-        let allocator: Arc<dyn TensorAllocator> = Arc::new(BitNetHipAllocator::new(Arc::clone(&ctx))?);
-        // provider.rs:87-99: the same twelve names, so that can_handle answers as before; the
-        // operations outside the ternary matmul fail at compile_subgraph with a message that says so
-        let supported_ops: HashSet<String> = [
-            "MatMul", "Gemm", "Conv", "Add", "Sub", "Mul", "And", "Or", "Xor", "BatchNormalization", "ReLU",
-            "Sigmoid",
-        ]
-        .iter()
-        .map(|s| s.to_string())
-        .collect();
-        info!("BitNet provider supports {} operations", supported_ops.len());
-        Ok(Self { config, ctx, allocator, supported_ops })
+        let c = config.to_c();
+        let mut raw = null_mut();
+        // SAFETY: valid in- and out-pointers.
+        check(unsafe { sys::rbp_provider_create(&c, &mut raw) })?;
+        let handle = Arc::new(ProviderHandle { raw });
+        let allocator: Arc<dyn TensorAllocator> = Arc::new(BitNetHipAllocator { provider: Arc::clone(&handle) });
+        Ok(Self { handle, allocator })
     }
 
-    pub fn get_config(&self) -> &BitNetProviderConfig {
-        &self.config
+    /// provider.rs:117-119 (by value: the configuration lives in the library).
+    pub fn get_config(&self) -> BitNetProviderConfig {
+        // SAFETY: plain-old-data out-parameter.
+        let mut c: sys::rbp_config = unsafe { std::mem::zeroed() };
+        let _ = unsafe { sys::rbp_provider_get_config(self.handle.raw, &mut c) };
+        BitNetProviderConfig::from_c(&c)
     }
 
+    /// provider.rs:121-123.
+    pub fn get_memory_stats(&self) -> BitNetMemoryStats {
+        let (mut binary, mut ternary, mut saved, mut ratio) = (0u64, 0u64, 0u64, 1f32);
+        // SAFETY: valid out-pointers.
+        let _ = unsafe {
+            sys::rbp_provider_memory_stats(self.handle.raw, &mut binary, &mut ternary, &mut saved, &mut ratio)
+        };
+        BitNetMemoryStats {
+            binary_tensor_count: binary as usize,
+            ternary_tensor_count: ternary as usize,
+            memory_saved_bytes: saved as usize,
+            average_compression_ratio: ratio,
+        }
+    }
+
+    /// provider.rs:127-129.
     pub fn supports_operation(&self, op_type: &str) -> bool {
-        self.supported_ops.contains(op_type)
+        match CString::new(op_type) {
+            // SAFETY: NUL-terminated string that outlives the call.
+            Ok(name) => unsafe { sys::rbp_provider_supports(self.handle.raw, name.as_ptr()) == 1 },
+            Err(_) => false,
+        }
     }
 
-    /// provider.rs:132-150, the same constants.
+    /// provider.rs:132-150.
     pub fn estimate_speedup(&self, op_spec: &OperatorSpec) -> f32 {
-        match op_spec.op_type.as_str() {
-            "MatMul" | "Gemm" => match self.config.quantization_method {
-                QuantizationMethod::Binary => 64.0,
-                QuantizationMethod::Ternary => 32.0,
-                QuantizationMethod::AsymmetricBinary { .. } => 48.0,
-            },
-            "Conv" => match self.config.quantization_method {
-                QuantizationMethod::Binary => 32.0,
-                QuantizationMethod::Ternary => 24.0,
-                QuantizationMethod::AsymmetricBinary { .. } => 28.0,
-            },
-            "Add" | "Sub" | "Mul" => 16.0,
-            "And" | "Or" | "Xor" => 128.0,
-            _ => 4.0,
+        match CString::new(op_spec.op_type.as_str()) {
+            // SAFETY: as above.
+            Ok(name) => unsafe { sys::rbp_provider_estimate_speedup(self.handle.raw, name.as_ptr()) },
+            Err(_) => 4.0,
         }
     }
 
-    /// provider.rs:153-210.  MatMul / Gemm with the ternary method get the GPU kernel, which
-    /// takes m, n, k from its inputs (the reference fixes them at 64).
-    fn create_kernel_for_operation(&self, node: &GraphNode) -> Result<Box<dyn CompiledKernel>> {
-        match node.op_type.as_str() {
-            "MatMul" | "Gemm" => match self.config.quantization_method {
-                QuantizationMethod::Ternary => Ok(Box::new(HipTernaryMatMul::new(
-                    Arc::clone(&self.ctx),
-                    self.config.strict_reference_sum,
-                    self.config.activation,
-                    self.config.max_cache_size,
-                ))),
-                _ => Err(anyhow!(
-                    "Binary (XNOR) kernels are not part of the MI355X BitNet provider: configure quantization_method = ternary"
-                )),
-            },
-            "And" | "Or" | "Xor" | "Add" | "Sub" | "Mul" | "Conv" | "ReLU" | "BatchNormalization" => Err(anyhow!(
-                "Operation {} runs on binary kernels, which are not part of the MI355X BitNet provider",
-                node.op_type
-            )),
-            _ => Err(anyhow!("Unsupported operation for BitNet: {}", node.op_type)), // provider.rs:205-208
-        }
+    /// `create_ternary_matmul_kernel(m, n, k)` (kernels.rs:339-344) on this provider's device;
+    /// 0, 0, 0 takes the dimensions from the inputs of each call.
+    pub fn create_ternary_matmul_kernel(&self, m: usize, n: usize, k: usize) -> Result<HipKernel> {
+        let mut raw = null_kernel();
+        // SAFETY: valid out-pointer.
+        check(unsafe { sys::rbp_create_ternary_matmul_kernel(self.handle.raw, m as u64, n as u64, k as u64, &mut raw) })?;
+        Ok(HipKernel::from_raw(raw))
     }
 }
 
@@ -235,9 +261,16 @@ impl ExecutionProvider for BitNetExecutionProvider {
 
     /// provider.rs:250-271 with the memory type of this implementation.
     fn get_capability(&self) -> ProviderCapability {
+        let supported_ops: HashSet<String> =
+            OP_NAMES.iter().filter(|op| self.supports_operation(op)).map(|op| op.to_string()).collect();
+        let data_types = [DataType::Bool, DataType::U8, DataType::F32, DataType::F16]
+            .into_iter()
+            // SAFETY: pure query.
+            .filter(|&dt| unsafe { sys::rbp_provider_has_data_type(self.handle.raw, dtype_to_code(dt)) } == 1)
+            .collect();
         ProviderCapability {
-            supported_ops: self.supported_ops.clone(),
-            data_types: vec![DataType::Bool, DataType::U8, DataType::F32, DataType::F16],
+            supported_ops,
+            data_types,
             memory_types: vec![MemoryType::DeviceMemory],
             performance_profile: PerformanceProfile::MemoryOptimized,
             resource_requirements: ResourceRequirements {
@@ -252,87 +285,65 @@ impl ExecutionProvider for BitNetExecutionProvider {
         operators.iter().map(|op| self.supports_operation(&op.op_type)).collect()
     }
 
-    /// provider.rs:280-310.  The reference's cache lookup can only fail ("Kernel caching not
-    /// fully implemented", :289-293, on a map that is never filled); there is no such map here:
-    /// what is worth caching - the ternarised weights - is cached inside the kernel.
+    /// provider.rs:280-310.  The single-node rule and the messages for unsupported operations
+    /// ("BitNet provider currently supports only single-node subgraphs", "Unsupported operation
+    /// for BitNet: {op}") are the library's.  The reference's cache lookup can only fail (:289-293,
+    /// on a map that is never filled); what is worth caching - the ternarised weights - is cached
+    /// inside the kernel object.
     fn compile_subgraph(&self, subgraph: SubGraph) -> Result<Box<dyn CompiledKernel>> {
         debug!("Compiling BitNet subgraph with {} nodes", subgraph.nodes.len());
-        if subgraph.nodes.len() != 1 {
-            return Err(anyhow!("BitNet provider currently supports only single-node subgraphs"));
-        }
-        let node = &subgraph.nodes[0];
-        let kernel = self.create_kernel_for_operation(node)?;
-        info!("Successfully compiled BitNet kernel for {}", node.op_type);
-        Ok(kernel)
+        let names: Vec<CString> = subgraph
+            .nodes
+            .iter()
+            .map(|node| CString::new(node.op_type.as_str()).map_err(|_| anyhow!("operation name contains NUL")))
+            .collect::<Result<_>>()?;
+        let ptrs: Vec<*const c_char> = names.iter().map(|n| n.as_ptr()).collect();
+        let mut raw = null_kernel();
+        // SAFETY: `ptrs` has `ptrs.len()` NUL-terminated strings that outlive the call.
+        check(unsafe { sys::rbp_provider_compile_subgraph(self.handle.raw, ptrs.as_ptr(), ptrs.len() as c_int, &mut raw) })?;
+        info!("Successfully compiled BitNet kernel for {}", subgraph.nodes[0].op_type);
+        Ok(Box::new(HipKernel::from_raw(raw)))
     }
 
     fn get_allocator(&self) -> Arc<dyn TensorAllocator> {
         Arc::clone(&self.allocator)
     }
 
-    /// provider.rs:316-364.  `custom_options` are applied at every optimisation level (the
-    /// reference parses them only under `Custom`, although its own test sets them under
-    /// `Aggressive`, provider.rs:479-500); two keys are new: `activation` = ternary | int8 and
-    /// `strict_reference_sum` = true | false.
+    /// provider.rs:316-364.  The library applies `custom_options` at every optimisation level
+    /// (the reference parses them only under `Custom`, although its own test sets them under
+    /// `Aggressive`, provider.rs:479-500) and knows two more keys: `activation` = ternary | int8
+    /// and `strict_reference_sum` = true | false.
     fn configure(&mut self, config: ProviderConfig) -> Result<()> {
-        if let Some(memory_limit) = config.memory_limit {
-            self.config.max_cache_size = (memory_limit / 4).min(128 * 1024 * 1024);
-        }
-        match config.optimization_level {
-            OptimizationLevel::None => {
-                self.config.memory_optimization_level = 0;
-                self.config.enable_simd = false;
-            }
-            OptimizationLevel::Basic => {
-                self.config.memory_optimization_level = 1;
-                self.config.enable_simd = true;
-            }
-            OptimizationLevel::Aggressive => {
-                self.config.memory_optimization_level = 2;
-                self.config.enable_simd = true;
-                self.config.enable_mixed_precision = true;
-            }
-            OptimizationLevel::Custom => {}
-        }
-        for (key, value) in &config.custom_options {
-            match key.as_str() {
-                "quantization_method" => {
-                    self.config.quantization_method = match value.as_str() {
-                        "binary" => QuantizationMethod::Binary,
-                        "ternary" => QuantizationMethod::Ternary,
-                        _ => QuantizationMethod::Binary,
-                    };
-                }
-                "enable_mixed_precision" => {
-                    self.config.enable_mixed_precision = value.parse().unwrap_or(true);
-                }
-                "enable_simd" => {
-                    self.config.enable_simd = value.parse().unwrap_or(true);
-                }
-                "activation" => {
-                    self.config.activation = match value.as_str() {
-                        "int8" => ActivationMode::Int8PerToken,
-                        _ => ActivationMode::TernaryPerTensor,
-                    };
-                }
-                "strict_reference_sum" => {
-                    self.config.strict_reference_sum = value.parse().unwrap_or(true);
-                }
-                _ => warn!("Unknown BitNet config option: {}", key),
-            }
-        }
+        let level = match config.optimization_level {
+            OptimizationLevel::None => 0,
+            OptimizationLevel::Basic => 1,
+            OptimizationLevel::Aggressive => 2,
+            OptimizationLevel::Custom => 3,
+        };
+        let pairs: Vec<(CString, CString)> = config
+            .custom_options
+            .iter()
+            .filter_map(|(k, v)| Some((CString::new(k.as_str()).ok()?, CString::new(v.as_str()).ok()?)))
+            .collect();
+        let keys: Vec<*const c_char> = pairs.iter().map(|p| p.0.as_ptr()).collect();
+        let values: Vec<*const c_char> = pairs.iter().map(|p| p.1.as_ptr()).collect();
+        // SAFETY: both arrays have `pairs.len()` NUL-terminated strings that outlive the call.
+        check(unsafe {
+            sys::rbp_provider_configure(self.handle.raw, config.memory_limit.unwrap_or(0) as u64, level, keys.as_ptr(),
+                                        values.as_ptr(), pairs.len() as c_int)
+        })?;
         info!("BitNet provider reconfigured with optimization level: {:?}", config.optimization_level);
         Ok(())
     }
 
-    /// provider.rs:366-385.
+    /// provider.rs:366-385: reports the allocator's counters and waits for the device.
     fn shutdown(&self) -> Result<()> {
         info!("Shutting down BitNet execution provider");
         let memory_info = self.allocator.get_memory_info();
         info!("  Memory allocated: {} bytes", memory_info.allocated_bytes);
         info!("  Peak memory: {} bytes", memory_info.peak_bytes);
-        // SAFETY: the context is alive as long as `self`.
-        sys::check(unsafe { sys::rbn_sync(self.ctx.raw()) }).map_err(|m| anyhow!(m))
+        // SAFETY: the provider is alive as long as `self`.
+        check(unsafe { sys::rbp_provider_shutdown(self.handle.raw) })
     }
 }
 
@@ -351,7 +362,7 @@ mod tests {
     //! The reference's own provider tests (provider.rs:400-504) restated for this provider; they
     //! need a gfx950 device.
     use super::*;
-    use ronn_core::{Tensor, TensorLayout};
+    use ronn_core::{GraphNode, Tensor, TensorLayout};
     use std::collections::HashMap;
 
     fn ternary() -> BitNetProviderConfig {
@@ -394,6 +405,32 @@ mod tests {
         let bits: Vec<u32> = out[0].to_vec()?.iter().map(|v| v.to_bits()).collect();
         assert_eq!(bits, vec![0x404f3333, 0x00000000, 0xc04f3333, 0xc04f3333]); // +-3.2375
         assert_eq!(kernel.get_performance_stats().execution_count, 1);
+        Ok(())
+    }
+
+    #[test]
+    fn group_of_three_projections_is_one_launch() -> Result<()> {
+        // q/k/v: three weight matrices, one input row; each result equals an execute() of its own
+        let p = BitNetExecutionProvider::with_config(ternary())?;
+        let kernel = p.create_ternary_matmul_kernel(0, 0, 0)?;
+        let (k, n) = (64usize, 32usize);
+        let a = Tensor::from_data((0..k).map(|i| ((i * 37 % 17) as f32 - 8.0) * 0.25).collect(), vec![1, k],
+                                  DataType::F32, TensorLayout::RowMajor)?;
+        let bs: Vec<Tensor> = (0..3)
+            .map(|j| {
+                Tensor::from_data((0..k * n).map(|i| (((i * 31 + j * 7) % 23) as f32 - 11.0) * 0.01).collect(),
+                                  vec![k, n], DataType::F32, TensorLayout::RowMajor)
+            })
+            .collect::<Result<_>>()?;
+        let pairs: Vec<(&Tensor, &Tensor)> = bs.iter().map(|b| (&a, b)).collect();
+        let (outs, launches) = kernel.execute_group(&pairs)?;
+        assert_eq!(launches, 1);
+        for (b, got) in bs.iter().zip(&outs) {
+            let single = kernel.execute(&[a.clone(), b.clone()])?;
+            let want: Vec<u32> = single[0].to_vec()?.iter().map(|v| v.to_bits()).collect();
+            let bits: Vec<u32> = got.to_vec()?.iter().map(|v| v.to_bits()).collect();
+            assert_eq!(bits, want);
+        }
         Ok(())
     }
 }

@@ -43,6 +43,11 @@ def test_bitnet_provider_creation(provider):                      # provider.rs:
     assert not provider.supports_operation("LSTM")
 
 
+def test_memory_stats_start_empty(provider):                      # provider.rs:121-123, allocator.rs:168-175
+    assert provider.get_memory_stats() == {"binary_tensor_count": 0, "ternary_tensor_count": 0,
+                                           "memory_saved_bytes": 0, "average_compression_ratio": 1.0}
+
+
 def test_provider_capabilities(provider):                         # provider.rs:418-432
     cap = provider.get_capability()
     assert "MatMul" in cap["supported_ops"] and "And" in cap["supported_ops"]

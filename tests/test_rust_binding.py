@@ -41,7 +41,12 @@ def test_sys_crate_declares_every_entry_point_with_the_same_arity():
     declared = {}
     for prefix, path in HEADERS:
         declared.update(c_declarations(path, prefix))
-    assert len(declared) >= 85
+    assert len(declared) >= 88
+    # calibration probes and the cycle-stamp read-out are measuring aids of bench.py: the Rust
+    # crates neither bind nor call them
+    aids = {n for n in declared if n.startswith("rbn_probe_") or n.startswith("rbn_debug_")}
+    assert not aids & set(rust), "measuring aids bound in lib.rs: %s" % sorted(aids & set(rust))
+    declared = {n: p for n, p in declared.items() if n not in aids}
     missing = sorted(set(declared) - set(rust))
     extra = sorted(set(rust) - set(declared) - {"rbn_last_error", "rbp_last_error"})
     assert not missing, "not bound in lib.rs: %s" % missing
@@ -102,14 +107,22 @@ def test_provider_crate_uses_only_bound_symbols():
         text = open(os.path.join(ROOT, "rust", "ronn-providers-bitnet-hip", "src", f)).read()
         used = set(re.findall(r"sys::(rb[np]_[a-z0-9_]+)\s*\(", text))
         assert used and used <= bound, (f, used - bound)
+        # one host implementation: the crate forwards to the provider-level objects that the GPU
+        # tests exercise (rbp_*) and carries no second weight cache over the kernel-level calls
+        assert all(u.startswith("rbp_") for u in used), (f, sorted(u for u in used if not u.startswith("rbp_")))
         # the traits of crates/ronn-core/src/types.rs:153-213,294-303 are implemented in full
     prov = open(os.path.join(ROOT, "rust", "ronn-providers-bitnet-hip", "src", "provider.rs")).read()
     for method in ("provider_id", "get_capability", "can_handle", "compile_subgraph", "get_allocator", "configure",
                    "shutdown", "allocate", "deallocate", "get_memory_info"):
         assert re.search(r"fn %s\(" % method, prov), method
     kern = open(os.path.join(ROOT, "rust", "ronn-providers-bitnet-hip", "src", "hip_kernel.rs")).read()
-    for method in ("execute", "get_memory_usage", "get_performance_stats"):
+    for method in ("execute", "execute_group", "get_memory_usage", "get_performance_stats"):
         assert re.search(r"fn %s\(" % method, kern), method
+    for call in ("rbp_kernel_execute", "rbp_kernel_execute_group", "rbp_kernel_stats", "rbp_kernel_memory_usage"):
+        assert "sys::%s(" % call in kern, call
+    for call in ("rbp_provider_create", "rbp_provider_compile_subgraph", "rbp_provider_configure",
+                 "rbp_provider_memory_stats", "rbp_allocate", "rbp_deallocate"):
+        assert "sys::%s(" % call in prov, call
 
 
 def test_reference_patch_applies(tmp_path):

@@ -261,9 +261,10 @@ int rbn_skinny_launch_shape(uint64_t M, uint64_t K, uint64_t N, int32_t shape[8]
  * A shape whose launch would need more than RBN_STATIC_SCRATCH_TILES partial tiles of 16 x 64
  * int32 (ceil(N/64) * splits * ceil(M/16), only when the matrix is narrow enough to be split
  * along k; M <= 16 always fits) is refused with RBN_ERR_UNSUPPORTED and a message that names
- * the need and the limit.  All calls on one GPU share the array, from whichever context:
- * calls that overlap on one GPU race and give wrong results; calls on one context are
- * serialised by the context's lock and stream. */
+ * the need and the limit.  All calls on one GPU share the array: calls that overlap on one GPU
+ * would race, so the first context that calls this entry point on a GPU holds the array until
+ * that context is destroyed (calls on one context are serialised by its lock and stream) and
+ * a call from any other context on that GPU is refused with RBN_ERR_INVALID. */
 #define RBN_STATIC_SCRATCH_TILES 1024
 #define RBN_STATIC_SCRATCH_BYTES (RBN_STATIC_SCRATCH_TILES * 4096 + 128 * 4)
 int rbn_gemm_t2_i8_skinny_static(rbn_ctx *ctx, const int8_t *d_q, const float *d_act_scale,

@@ -50,6 +50,8 @@ void rbn_clear_error();
 // Per-device set-up of the small-batch kernels (dynamic-LDS limit, address of their static
 // scratch array); called with `device` current.
 int rbn_skinny_prepare(int device);
+// gives up the context's claim on its GPU's static scratch array (rbn_ctx_destroy)
+void rbn_skinny_release(const rbn_ctx *ctx);
 
 // Ensures ctx->ws has at least `bytes` bytes; returns it through *out.
 int rbn_workspace(rbn_ctx *ctx, size_t bytes, void **out);

@@ -142,6 +142,7 @@ int rbn_ctx_destroy(rbn_ctx *ctx) {
     if (!ctx) return RBN_OK;
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    rbn_skinny_release(ctx);
     if (ctx->ws) (void)hipFree(ctx->ws);
     if (ctx->ws2) (void)hipFree(ctx->ws2);
     if (ctx->mailbox) (void)hipHostFree(ctx->mailbox);
@@ -245,6 +246,7 @@ int rbn_sync(rbn_ctx *ctx) {
 int rbn_device_flags(rbn_ctx *ctx, uint32_t *h_flags) {
     RBN_ENTER(ctx);
     RBN_REQUIRE(h_flags != nullptr, "h_flags is NULL");
+    RBN_CHECK(rbn_refuse_while_capturing(ctx, "rbn_device_flags"));
     unsigned *box = static_cast<unsigned *>(ctx->mailbox) + 512;  // the mailbox's second half
     RBN_HIP(hipMemcpyAsync(box, ctx->dev_flags, sizeof(unsigned), hipMemcpyDeviceToHost, ctx->stream));
     fill_u8_kernel<<<dim3(1), dim3(64), 0, ctx->stream>>>((uint8_t *)ctx->dev_flags, 0, sizeof(unsigned));

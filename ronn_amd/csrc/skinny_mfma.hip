@@ -628,6 +628,16 @@ static __device__ __align__(256) unsigned char scratch[kStaticBytes];
 constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_lock;
 static void *g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, 0 until prepared
+// The context that uses a GPU's static scratch: the first one to call the entry point, until it
+// is destroyed.  Calls from two contexts would run on two streams and corrupt each other's
+// partial tiles and counters, so a second context is refused instead.
+static const rbn_ctx *g_scratch_owner[kMaxDevices];
+
+void rbn_skinny_release(const rbn_ctx *ctx) {
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    for (int d = 0; d < kMaxDevices; ++d)
+        if (g_scratch_owner[d] == ctx) g_scratch_owner[d] = nullptr;
+}
 
 __global__ void clear_tickets_kernel(unsigned *tickets, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -864,12 +874,20 @@ extern "C" int rbn_gemm_t2_i8_skinny_static(rbn_ctx *ctx, const int8_t *d_q, con
                                             int32_t *d_acc, float *d_out) {
     RBN_ENTER(ctx);
     void *base = nullptr;
+    bool mine = true;
     if (ctx->device >= 0 && ctx->device < kMaxDevices) {
         std::lock_guard<std::mutex> hold(g_scratch_lock);
         base = g_scratch_ptr[ctx->device];
+        if (g_scratch_owner[ctx->device] == nullptr) g_scratch_owner[ctx->device] = ctx;
+        mine = g_scratch_owner[ctx->device] == ctx;
     }
     if (base == nullptr)
         return rbn_fail(RBN_ERR_HIP, "the static scratch of device %d was never looked up", ctx->device);
+    if (!mine)
+        return rbn_fail(RBN_ERR_INVALID,
+                        "the static scratch of device %d is in use by another context: one context per GPU "
+                        "may call rbn_gemm_t2_i8_skinny_static (it is released when that context is destroyed)",
+                        ctx->device);
     unsigned *tickets = reinterpret_cast<unsigned *>(static_cast<unsigned char *>(base) +
                                                      (size_t)kStaticTiles * 4096);
     return skinny_impl(ctx, "rbn_gemm_t2_i8_skinny_static", d_q, d_act_scale, d_rowsum, d_tiled, w_scale, M,

@@ -42,6 +42,45 @@ def test_static_scratch_matches_on_consecutive_calls(ctx):
     both(ctx, 4, 1024, 16384, 9)
 
 
+def test_static_call_under_graph_capture_allocates_nothing(ctx):
+    # captured in a HIP graph (where an allocation would be an error) and replayed three times with
+    # eager work in between: every replay gives the eager entry point's bits, and the library's
+    # device-memory accounting does not move across capture and replays
+    M, K, N = 16, 11008, 512                     # split along k: partial tiles and tickets in the static array
+    acts, d_t, w_scale = operands(ctx, M, K, N, 21)
+    want_out, want_acc = ctx.skinny(acts, d_t, w_scale, M, K, N, want_acc=True)
+    d_out, d_acc = ctx.alloc(4 * M * N), ctx.alloc(4 * M * N)
+    ctx.sync()
+    before = ctx.memory_info()
+    ctx.graph_begin()
+    ctx.skinny_static(acts, d_t, w_scale, M, K, N, d_out=d_out, d_acc=d_acc)
+    graph = ctx.graph_end()
+    assert ctx.memory_info() == before
+    n = M * N
+    for replay in range(3):
+        ctx.lib.rbn_fill_u8(ctx.handle, d_out.ptr, 0xFF, 4 * n)
+        ctx.graph_launch(graph)
+        ctx.sync()
+        assert (d_acc.download(np.int32, n) == want_acc.download(np.int32, n)).all(), replay
+        assert (d_out.download(np.uint32, n) == want_out.download(np.uint32, n)).all(), replay
+        both(ctx, 8, 4096, 1024, 30 + replay)     # eager work on the same scratch between replays
+    assert ctx.memory_info()[0] >= before[0]      # (the eager calls above allocate their own operands)
+    ctx.graph_destroy(graph)
+
+
+def test_static_scratch_belongs_to_one_context_per_gpu(ctx):
+    # `ctx` has used the array above; another context on the same GPU is refused until `ctx` goes
+    from ronn_amd.device import Context
+    both(ctx, 8, 4096, 1024, 40)
+    with Context(0) as other:
+        d = other.alloc(65536)
+        rc = other.lib.rbn_gemm_t2_i8_skinny_static(other.handle, d.ptr, d.ptr, d.ptr, d.ptr, 1.0, 1, 64, 64, None,
+                                                    d.ptr)
+        assert rc == _lib.RBN_ERR_INVALID
+        assert "in use by another context" in other.lib.rbn_last_error().decode()
+    both(ctx, 8, 4096, 1024, 41)
+
+
 def test_static_scratch_refuses_what_does_not_fit(ctx):
     # 127 column groups x 3 parts x 4 row tiles = 1524 partial tiles > 1024: refused on the
     # host, nothing is launched

@@ -395,13 +395,22 @@ __device__ __forceinline__ void wait_vm() {
 
 constexpr int kStageUnits = 256;  // 16-byte units of one stage: weights 0-127, activations 128-255
 
-template <int D, bool REFILL>
+// HALF: at most eight tokens - the transfer of tokens 8-15 is left out (their rows of the stage
+// keep whatever LDS held; the MFMA rows they feed are never stored).  WHALF: the workgroup owns at
+// most eight column quads - the transfer of quads 8-15 is left out likewise (their columns are never
+// stored).
+// A workgroup owns the quads [group * nquads / groups, (group + 1) * nquads / groups): sixteen when
+// there are at least as many groups of sixteen as the launch wants workgroups, fewer when the host
+// spreads a narrower matrix over more workgroups so that every CU streams a share of the weights
+// (what one CU can keep in flight is a quarter of a megabyte per microsecond or so; 4096 x 11008 on
+// 172 workgroups of sixteen quads gave each CU 64 KiB to pull, on 256 workgroups 43 KiB).
+template <int D, bool REFILL, bool HALF, bool WHALF>
 __global__ __launch_bounds__(1024) void skinny_dma_kernel(
     const int8_t *__restrict__ q,         // [M][Kpad], Kpad % 128 == 0, M <= 16
     const float *__restrict__ act_scale, const int32_t *__restrict__ rowsum,
     const uint4 *__restrict__ wt,         // tiled: uint4 index quad * KB + kb
-    float w_scale, int M, int Kpad, int N, int groups, int splits,
-    int4 *__restrict__ partials, unsigned *__restrict__ tickets,
+    float w_scale, int M, int Kpad, int N, int nquads /* of the tiled buffer: a multiple of 16 */, int groups,
+    int splits, int4 *__restrict__ partials, unsigned *__restrict__ tickets,
     int32_t *__restrict__ acc_out, float *__restrict__ out) {
     extern __shared__ uint4 ring[];  // [waves][D][kStageUnits]; reused as [waves][256] int4 for the join
     __shared__ int s_last;
@@ -417,19 +426,38 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
     const int group = blockIdx.x % groups, split = blockIdx.x / groups;
     const int gw = split * nw + wave, gn = splits * nw;
     const int s0 = gw * stages / gn, s1 = (gw + 1) * stages / gn;  // >= 1 stage (the host sees to it)
+    // this workgroup's quads: 1 to 16 of them (the host keeps nquads / groups within that)
+    const int q_lo = (int)(((long long)group * nquads) / groups);
+    const int nq = min(max((int)(((long long)(group + 1) * nquads) / groups) - q_lo, 1), 16);
 
     // transfer h of a stage: row (quad or token) 8h + lane/8, slot lane%8 holding k-block
-    // slot ^ ((row>>1)&7) of the stage's eight
+    // slot ^ ((row>>1)&7) of the stage's eight; rows past the workgroup's quads or the tokens that
+    // exist repeat the last one (fetched again, never stored)
     const int sub = lane >> 3, slot = lane & 7;
     uint32_t w_off[2], a_off[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
         const int row = 8 * h + sub;
         const int kb = slot ^ ((row >> 1) & 7);
-        w_off[h] = ((uint32_t)row * (uint32_t)KB + (uint32_t)kb) * 16u;
+        w_off[h] = ((uint32_t)min(row, nq - 1) * (uint32_t)KB + (uint32_t)kb) * 16u;
         a_off[h] = (uint32_t)min(row, M - 1) * (uint32_t)Kpad + (uint32_t)kb * 16u;
     }
-    const uint4 *w_base = wt + (size_t)group * 16 * KB;  // the group's sixteen quads exist (N is padded to 64)
+    const uint4 *w_base = wt + (size_t)min(q_lo, nquads - 1) * KB;
+    // The epilogue's per-token scalars, asked for before the transfers (the memory counter retires in
+    // order, and the hand-counted waits below count transfers only): a thread finishes the elements
+    // tid, tid + blockDim.x, ... of the 16 x 16 tile, element e belonging to token e / 16.  Fetched at the
+    // end they were a dependent round trip after the join barrier.
+    int rs_pre[4] = {0, 0, 0, 0};
+    float as_pre[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {  // a workgroup of one wave finishes four elements per thread, of four or more one
+        const int idx = tid + j * (int)blockDim.x;
+        if (idx < 256) {
+            const int row = min(idx >> 4, M - 1);
+            rs_pre[j] = rowsum[row];
+            as_pre[j] = act_scale[row];
+        }
+    }
     const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr)ring + (uint32_t)wave * (D * kStageUnits * 16);
     auto issue = [&](int s, int d) {
         // past the range: a re-read of the last stage, multiplied by zero (and never below stage 0,
@@ -439,10 +467,11 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
         const int8_t *ab = q + (size_t)sc * 128;
         const uint32_t at = lds0 + (uint32_t)d * (kStageUnits * 16);
         dma16(wb, w_off[0], at);
-        dma16(wb, w_off[1], at + 1024);
+        if (!WHALF) dma16(wb, w_off[1], at + 1024);
         dma16(ab, a_off[0], at + 2048);
-        dma16(ab, a_off[1], at + 3072);
+        if (!HALF) dma16(ab, a_off[1], at + 3072);
     };
+    constexpr int LPS = 4 - (HALF ? 1 : 0) - (WHALF ? 1 : 0);  // transfers per stage
 #pragma unroll
     for (int d = 0; d < D; ++d) issue(s0 + d, d);
     SK_STAMP(1);
@@ -477,7 +506,7 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
         // transfers are outstanding
         auto step = [&](auto dt) {
             constexpr int d = decltype(dt)::value;
-            wait_vm<4 * (D - 1 - d)>();
+            wait_vm<LPS * (D - 1 - d)>();
             consume(d, s0 + d < s1 ? 0xffffffffu : 0u);
         };
         step(std::integral_constant<int, 0>{});
@@ -491,7 +520,7 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
         do {
             auto step = [&](auto dt) {
                 constexpr int d = decltype(dt)::value;
-                wait_vm<4 * (D - 1)>();
+                wait_vm<LPS * (D - 1)>();
                 consume(d, base + d < s1 ? 0xffffffffu : 0u);
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 issue(base + d + D, d);
@@ -518,12 +547,12 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
     SK_STAMP(3);
 
     const bool vec_ok = (N & 3) == 0;
-    auto finish = [&](int idx, int4 t) {
+    auto finish = [&](int idx, int j, int4 t) {  // idx = tid + j * blockDim.x
         const int row = idx / quads, qd = idx - row * quads;
-        const int col0 = (group * quads + qd) * 4;
-        if (row >= M || col0 >= N) return;
-        const int rs = rowsum[row];
-        const float as = act_scale[row];
+        const int col0 = (q_lo + qd) * 4;
+        if (row >= M || qd >= nq || col0 >= N) return;
+        const int rs = rs_pre[j];
+        const float as = as_pre[j];
         const int ti[4] = {t.x - rs, t.y - rs, t.z - rs, t.w - rs};
         float v[4];
 #pragma unroll
@@ -547,7 +576,10 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
     };
 
     int4 *my_part = partials + ((size_t)group * splits + split) * tile;
-    for (int idx = tid; idx < tile; idx += blockDim.x) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int idx = tid + j * (int)blockDim.x;
+        if (idx >= tile) break;
         int4 t = red[idx];
         for (int w = 1; w < nw; ++w) {
             const int4 p = red[w * wstride + idx];
@@ -557,7 +589,7 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
             t.w += p.w;
         }
         if (splits == 1)
-            finish(idx, t);
+            finish(idx, j, t);
         else
             store_device_scope(my_part + idx, t);
     }
@@ -582,7 +614,10 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
     __syncthreads();
     if (!s_last) return;
     const int4 *all = partials + (size_t)group * splits * tile;
-    for (int idx = tid; idx < tile; idx += blockDim.x) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int idx = tid + j * (int)blockDim.x;
+        if (idx >= tile) break;
         int4 t = make_int4(0, 0, 0, 0);
         for (int sp0 = 0; sp0 < splits; sp0 += 4) {
             int4 p[4];
@@ -597,23 +632,43 @@ __global__ __launch_bounds__(1024) void skinny_dma_kernel(
                 t.w += p[i].w & keep;
             }
         }
-        finish(idx, t);
+        finish(idx, j, t);
     }
 }
 
 template <int D, bool REFILL>
 int launch_dma(hipStream_t stream, const Args &a) {
     const size_t lds = (size_t)a.waves * D * kStageUnits * 16;
-    skinny_dma_kernel<D, REFILL><<<dim3((unsigned)(a.groups * a.splits)), dim3((unsigned)a.waves * 64), lds, stream>>>(
-        a.q, a.act_scale, a.rowsum, a.wt, a.w_scale, a.M, a.Kpad, a.N, a.groups, a.splits, a.partials, a.tickets,
-        a.acc, a.out);
+    const dim3 grid((unsigned)(a.groups * a.splits)), block((unsigned)a.waves * 64);
+    const int nquads = (int)(rbn_npad((uint64_t)a.N) / 4);
+    const bool half = a.M <= 8;                                   // no token beyond the eighth
+    const bool whalf = (nquads + a.groups - 1) / a.groups <= 8;   // no workgroup with more than eight quads
+    auto go = [&](auto kernel) {
+        kernel<<<grid, block, lds, stream>>>(a.q, a.act_scale, a.rowsum, a.wt, a.w_scale, a.M, a.Kpad, a.N, nquads,
+                                             a.groups, a.splits, a.partials, a.tickets, a.acc, a.out);
+    };
+    if (half && whalf)
+        go(skinny_dma_kernel<D, REFILL, true, true>);
+    else if (half)
+        go(skinny_dma_kernel<D, REFILL, true, false>);
+    else if (whalf)
+        go(skinny_dma_kernel<D, REFILL, false, true>);
+    else
+        go(skinny_dma_kernel<D, REFILL, false, false>);
     return RBN_OK;
 }
 
 template <int D, bool REFILL>
 hipError_t allow_large_lds_dma() {
-    return hipFuncSetAttribute(reinterpret_cast<const void *>(skinny_dma_kernel<D, REFILL>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+    const void *fns[] = {reinterpret_cast<const void *>(skinny_dma_kernel<D, REFILL, true, true>),
+                         reinterpret_cast<const void *>(skinny_dma_kernel<D, REFILL, true, false>),
+                         reinterpret_cast<const void *>(skinny_dma_kernel<D, REFILL, false, true>),
+                         reinterpret_cast<const void *>(skinny_dma_kernel<D, REFILL, false, false>)};
+    for (const void *f : fns) {
+        const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
 }
 
 }  // namespace
@@ -706,7 +761,7 @@ static bool plan_skinny(uint64_t M, uint64_t K, uint64_t N, int max_tiles, int m
     // the workgroups more than the saving (4096 x 11008: 18 us with one group, 28 with two)
     const int cgroups = (int)(rbn_npad(N) / 64);
     const int ng = (mt == 4 && cgroups >= 256) ? 2 : 1;
-    const int groups = (cgroups + ng - 1) / ng;
+    int groups = (cgroups + ng - 1) / ng;
     // Shape of the launch (measured on the decode shapes; 64-k steps per wave in brackets).
     // With enough column groups, one workgroup per group: 4096 x 11008 runs 16 waves [4],
     // 8192 x 28672 16 waves [8].  Narrower matrices are also split along k across
@@ -726,6 +781,22 @@ static bool plan_skinny(uint64_t M, uint64_t K, uint64_t N, int max_tiles, int m
         const int per = M <= 8 ? 48 : 32;
         const int want = (steps + per - 1) / per;
         if (want < splits) splits = want;
+    }
+    // Up to 16 tokens with a short k (the activation block is at most 64 KiB): where the rule above
+    // would split along k, the matrix is cut along N instead, into up to 256 workgroups of four to
+    // sixteen quads (the kernel gives workgroup g the quads [g * nquads / groups, (g + 1) * nquads /
+    // groups)).  Every workgroup then reads the whole activation block, but nothing is exchanged
+    // through memory: 4096 x 4096 5.6-5.9 -> 5.2-5.5 us, 2560 x 7680 and 2560 x 2560 at 16 tokens
+    // 5.7 -> 5.0 and 5.2 -> 4.5 us.  With a longer k the activation traffic of that many workgroups
+    // outweighs the exchange (11008 x 4096: 7.1 -> 8.3-9.5 us), and a matrix that needs no split gains
+    // nothing from more workgroups (4096 x 11008 on 256 instead of 172: 5.9 -> 6.2 us).
+    if (mt == 1 && splits > 1 && Kpad <= 4096) {
+        const int nquads = cgroups * 16;
+        int wide = nquads / 4 < 256 ? nquads / 4 : 256;
+        if (wide > groups) {
+            groups = wide;
+            splits = 1;
+        }
     }
     // the exchange area holds max_tiles tiles of 16 x 64 int32 and one ticket per group
     bool fits = true;

@@ -260,6 +260,10 @@ def test_small_batch_launch_shapes_meet_the_kernels_assumptions(lib):
                 assert longest == -(-steps // (splits * waves)) and longest >= 1
                 assert 0 < lds <= 128 * 1024
                 assert groups >= 1 and groups * 64 * (2 if (M > 32 and -(-N // 64) >= 256) else 1) >= N
+                if ring:
+                    # workgroup g owns the quads [g*nquads/groups, (g+1)*nquads/groups): 1 to 16 of them
+                    nquads = -(-N // 64) * 16
+                    assert groups <= nquads and -(-nquads // groups) <= 16 and groups <= max(256, nquads // 16)
                 # the partition the kernels use: wave w of g takes steps [w*steps/g, (w+1)*steps/g)
                 g = splits * waves
                 assert all((w + 1) * steps // g > w * steps // g for w in range(g))
@@ -273,4 +277,10 @@ def test_small_batch_launch_shapes_meet_the_kernels_assumptions(lib):
     lib.rbn_skinny_launch_shape(16, 4096, 11008, shape)
     assert list(shape)[:7] == [1, 172, 1, 16, 128, 32, 2]
     lib.rbn_skinny_launch_shape(16, 4096, 4096, shape)
-    assert list(shape)[:4] == [1, 64, 2, 8]
+    assert list(shape)[:4] == [1, 256, 1, 16]                # four quads each instead of a split along k
+    lib.rbn_skinny_launch_shape(16, 11008, 4096, shape)
+    assert list(shape)[:3] == [1, 64, 4]                     # long k: split along k, sixteen quads each
+    lib.rbn_skinny_launch_shape(4, 2560, 2560, shape)
+    assert list(shape)[:3] == [1, 40, 1]
+    lib.rbn_skinny_launch_shape(8, 8192, 28672, shape)
+    assert list(shape)[:4] == [1, 448, 1, 16]                # wide enough: sixteen quads each, as before

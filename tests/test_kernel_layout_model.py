@@ -46,7 +46,8 @@ def decode_b(word):
     return np.array([(word >> (8 * b + 2 * s)) & 3 for s in range(4) for b in range(4)], dtype=np.int64)
 
 
-@pytest.mark.parametrize("M,K,N", [(16, 256, 64), (5, 384, 130), (16, 1100, 64), (3, 128, 37), (9, 4096, 64)])
+@pytest.mark.parametrize("M,K,N", [(16, 256, 64), (5, 384, 130), (16, 1100, 64), (3, 128, 37), (9, 4096, 64),
+                                   (16, 256, 704), (8, 128, 1100), (12, 256, 2752)])
 def test_lds_ring_kernel_model(lib, M, K, N):
     rng = np.random.default_rng(M * 1000 + K + N)
     vals = rng.integers(-1, 2, size=(K, N)).astype(np.int8)
@@ -66,16 +67,28 @@ def test_lds_ring_kernel_model(lib, M, K, N):
     assert lds_bytes == nw * D * 4096
 
     acc_total = np.zeros((groups, 16, 64), dtype=np.int64)      # [group][token][column in group]
+    nquads = npad // 4
+    half = M <= 8                                    # the transfer of tokens 8-15 is left out
+    whalf = (nquads + groups - 1) // groups <= 8     # ... and that of quads 8-15
     lanes = np.arange(64)
     sub, slot = lanes >> 3, lanes & 7
     ql, g = lanes & 15, lanes >> 4
+    q_los, nqs = [], []
     for group in range(groups):
+        # the workgroup's quads: [group * nquads / groups, (group + 1) * nquads / groups)
+        q_lo = group * nquads // groups
+        nq = min(max((group + 1) * nquads // groups - q_lo, 1), 16)
+        assert (group + 1) * nquads // groups - q_lo == nq and q_lo + nq <= nquads
+        assert nq <= 8 or not whalf
+        q_los.append(q_lo)
+        nqs.append(nq)
         for split in range(splits):
             for wave in range(nw):
                 gw, gn = split * nw + wave, splits * nw
                 s0, s1 = gw * stages // gn, (gw + 1) * stages // gn
                 assert s1 > s0
-                lds = np.zeros((D, 4096), dtype=np.uint8)       # this wave's ring
+                # this wave's ring; it starts with whatever the last kernel left there
+                lds = rng.integers(0, 256, size=(D, 4096)).astype(np.uint8)
                 acc = np.zeros((64, 4, 4), dtype=np.int64)      # [lane][tile j][register i]
 
                 def issue(s, d):
@@ -83,13 +96,15 @@ def test_lds_ring_kernel_model(lib, M, K, N):
                     for h in range(2):
                         row = 8 * h + sub
                         kb = slot ^ ((row >> 1) & 7)
-                        w_off = (row * KB + kb) * 16 + (group * 16 * KB + sc * 8) * 16
+                        w_off = (np.minimum(row, nq - 1) * KB + kb) * 16 + (q_lo * KB + sc * 8) * 16
                         a_off = np.minimum(row, M - 1) * kpad + kb * 16 + sc * 128
                         assert w_off.min() >= 0 and w_off.max() + 16 <= tiled.size
                         assert a_off.min() >= 0 and a_off.max() + 16 <= qbytes.size
                         for l in range(64):                      # lane l's 16 bytes land at base + 16 l
-                            lds[d, h * 1024 + 16 * l:h * 1024 + 16 * l + 16] = tiled[w_off[l]:w_off[l] + 16]
-                            lds[d, 2048 + h * 1024 + 16 * l:2048 + h * 1024 + 16 * l + 16] = qbytes[a_off[l]:a_off[l] + 16]
+                            if not (h == 1 and whalf):
+                                lds[d, h * 1024 + 16 * l:h * 1024 + 16 * l + 16] = tiled[w_off[l]:w_off[l] + 16]
+                            if not (h == 1 and half):
+                                lds[d, 2048 + h * 1024 + 16 * l:2048 + h * 1024 + 16 * l + 16] = qbytes[a_off[l]:a_off[l] + 16]
 
                 def consume(d, keep):
                     for t in range(2):
@@ -131,7 +146,14 @@ def test_lds_ring_kernel_model(lib, M, K, N):
                     for j in range(4):
                         for i in range(4):
                             acc_total[group, 4 * g[l] + i, 4 * ql[l] + j] += acc[l, j, i]
-    got = acc_total.transpose(1, 0, 2).reshape(16, groups * 64)[:M, :N]
+    # finish(): quad qd of the tile is column quad q_lo + qd, stored when qd < nq (and the token exists)
+    got = np.full((16, npad), np.iinfo(np.int64).min, dtype=np.int64)
+    for group in range(groups):
+        for qd in range(nqs[group]):
+            c0 = (q_los[group] + qd) * 4
+            assert (got[:, c0:c0 + 4] == np.iinfo(np.int64).min).all()      # no column is written twice
+            got[:, c0:c0 + 4] = acc_total[group, :, 4 * qd:4 * qd + 4]
+    got = got[:M, :N]
     # weights are codes = value + 1: the kernel subtracts the token's sum of q in the epilogue
     want = q_src.astype(np.int64) @ vals.astype(np.int64)
     rowsum = q.astype(np.int64).sum(axis=1, keepdims=True)

@@ -348,7 +348,8 @@ def time_act_quant(ctx):
 
 def time_stream_floor(ctx):
     """What launches that compute nothing cost on this machine: an empty kernel, and kernels
-    that only read (the GEMV's access pattern) 4, 11, 22 and 59 MB from rotating addresses."""
+    that only read (the GEMV's access pattern) 4, 11, 22, 59, 181 and 362 MB from rotating addresses
+    (the last two are what 16 and 32 grouped GEMVs of the headline shape read in one launch)."""
     from ronn_amd import _lib
     lib, h = ctx.lib, ctx.handle
     ev, _ = replay(ctx, lambda first, n: [_lib.check(lib.rbn_probe_empty_launch(h)) for _ in range(n)], 64, 640, 64,
@@ -357,7 +358,7 @@ def time_stream_floor(ctx):
     pool_bytes = 768 << 20
     pool = ctx.alloc(pool_bytes)
     _lib.check(lib.rbn_fill_u8(h, pool.ptr, 0x55, pool_bytes))
-    for size in (4194304, 11272192, 22544384, 58720256):
+    for size in (4194304, 11272192, 22544384, 58720256, 16 * 11320324 // 16 * 16, 32 * 11320324 // 16 * 16):
         slots = pool_bytes // size
         row = {"bytes": size}
         for nt in (0, 1):
@@ -627,6 +628,8 @@ def main():
                                "so every GEMV streams from HBM; HIP-graph replay; the one-GEMV-per-launch figure is "
                                "extra.gemv_one_per_launch" % (GROUP, gw.n, gw.n * gw.tiled_bytes / 2**20),
                    "M": M, "K": K, "N": N, "gemvs_per_launch": GROUP, "weight_buffers": gw.n,
+                   "realistic_groups": "extra.gemv_realistic_groups: fraction of HBM peak at 1, 2, 3, 8 and 32 GEMVs "
+                                       "per launch, with the caller that reaches each",
                    "gemvs_timed": args.steps * GROUP,
                    "preheat": "0.25 s of the same launches during set-up, before the warm-up steps (clock ramp)",
                    "device": info["name"] or info["arch"], "arch": info["arch"],
@@ -665,12 +668,22 @@ def main():
                                         "GBps": bytes_per_gemv / (ev1 * 1e-3) / 1e9,
                                         "frac_hbm_peak": bytes_per_gemv / (ev1 * 1e-3) / 1e9 / HBM_PEAK_GBS}
         rows = []
-        for g in (2, 4, 8, 16, 32):
+        for g in (2, 3, 4, 8, 16, 32):
             evg, _ = replay(ctx, lambda first, n: gw.launch(first % gw.n, n), g, 16 * gw.n, 2 * gw.n,
                             max_units_per_graph=gw.n)
             rows.append({"gemvs_per_launch": g, "us_per_gemv": evg * 1e3,
                          "frac_hbm_peak": bytes_per_gemv / (evg * 1e-3) / 1e9 / HBM_PEAK_GBS})
         extra["gemv_group_size_sweep"] = rows
+        # which callers reach which group size: one MatMul node per execute() is 1; the same-input
+        # projections of one token that BitNetKernel::execute_group / rbp_kernel_execute_group run as one
+        # launch are 2 (gate, up) and 3 (q, k, v); 8 and more need several sequences or experts per call
+        by_g = {r["gemvs_per_launch"]: r for r in rows}
+        extra["gemv_realistic_groups"] = {
+            "1 (CompiledKernel::execute, one MatMul node)": extra["gemv_one_per_launch"]["frac_hbm_peak"],
+            "2 (gate/up through execute_group)": by_g[2]["frac_hbm_peak"],
+            "3 (q/k/v through execute_group)": by_g[3]["frac_hbm_peak"],
+            "8 (eight sequences or experts through execute_group)": by_g[8]["frac_hbm_peak"],
+            "32 (the headline step)": by_g[32]["frac_hbm_peak"]}
         # warm variant: one buffer, lives in L2 / Infinity Cache
         evw, _ = replay(ctx, lambda first, n: [gw.launch_single(0) for _ in range(n)], 32, 2048, 256,
                         max_units_per_graph=64)

@@ -90,8 +90,8 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
     constexpr int kLoads = 2 * MT + 2;           // LDS loads per wave and stage
     constexpr int kWaitStage = 0x0070 | kLoads;  // s_waitcnt vmcnt(kLoads) lgkmcnt(0)
     __shared__ __attribute__((aligned(16))) uint4 smem[3 * (kAUnits + kBUnits)];
-    __shared__ float s_scale[TM];
-    __shared__ int s_rowsum[TM];
+    __shared__ __attribute__((aligned(16))) float s_scale[TM];
+    __shared__ __attribute__((aligned(16))) int s_rowsum[TM];
     __shared__ int s_last;
 
     const int tid = threadIdx.x;
@@ -104,13 +104,18 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
     // a band of m tiles and let it walk the n tiles.
     // With splits > 1 (few tiles, see the launch) `splits` consecutive workgroups share a
     // tile and take consecutive ranges of K steps.
+    // every argument the set-up below needs, asked for in one go: left to the compiler, the scalar
+    // loads of the arguments were fetched where first used, five dependent round trips before the
+    // first transfer could be issued
+    asm volatile("" : : "s"(M), "s"(Kpad), "s"(N), "s"(nquads), "s"(m_tiles), "s"(n_tiles), "s"(splits), "s"(q),
+                 "s"(wt), "s"(act_scale), "s"(rowsum));
     int tile = blockIdx.x, split = 0;
-    if (splits > 1) {
+    if (MT == 1 && splits > 1) {  // 128-row tiles are never split along K
         tile = blockIdx.x / splits;
         split = blockIdx.x - tile * splits;
     }
     int bm, bn;
-    if ((m_tiles & 7) == 0 && splits == 1) {
+    if ((m_tiles & 7) == 0 && (MT == 2 || splits == 1)) {
         const int per = m_tiles >> 3;
         const int xcd = tile & 7, i = tile >> 3;
         bm = xcd * per + i % per;
@@ -122,19 +127,17 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
     const int m0 = bm * TM, n0 = bn * BN;
     const int q0 = n0 >> 2;
 
+    // The epilogue's per-row scalars are asked for here and written to LDS only after the first two
+    // stages are on their way: staged at once, their round trip stood between the kernel's start and
+    // its first transfer (2,700 cycles from start to the first transfer, 630 more to the first data).
+    v16i acc[MT][4];  // zeroed below, behind the first transfers
+    float pre_scale = 0.0f;
+    int pre_rowsum = 0;
     if (tid < TM) {
         const int row = m0 + tid;
-        s_scale[tid] = row < M ? act_scale[row] : 0.0f;
-        s_rowsum[tid] = row < M ? rowsum[row] : 0;
+        pre_scale = row < M ? act_scale[row] : 0.0f;
+        pre_rowsum = row < M ? rowsum[row] : 0;
     }
-
-    v16i acc[MT][4];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
     // Per-lane source addresses of the stage loads.  Load j of wave w fills the units
     // (4j + w) * 64 + lane: row (or quad) (4j + w) * 8 + lane / 8, slot lane % 8, and the
@@ -159,7 +162,7 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
     }
     // this workgroup's K steps: [it_lo, it_lo + iters)
     const int iters_all = Kpad / BK;
-    const int per_split = (iters_all + splits - 1) / splits;
+    const int per_split = MT == 2 ? iters_all : (iters_all + splits - 1) / splits;
     const int it_lo = split * per_split;
     const int iters = min(per_split, iters_all - it_lo);  // >= 1 (the launch sees to it)
     a_base += (size_t)it_lo * BK;
@@ -249,6 +252,17 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
     // then fill the pipeline: raw fragments of sub-steps 0 and 1, weights of 0 decoded
     issue(0, 0);
     issue(1, 1);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+    if (tid < TM) {
+        s_scale[tid] = pre_scale;
+        s_rowsum[tid] = pre_rowsum;
+    }
     __builtin_amdgcn_s_waitcnt(kWaitStage);
     __builtin_amdgcn_s_barrier();
     lds_reads(0, 0);
@@ -353,6 +367,45 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
     // 8*(r/4) + 4*(lane/32) + r%4 of each 32-row tile
     const int col0 = n0 + fquad * 4;
     const bool vec_ok = (N & 3) == 0;
+    // A tile that lies inside the matrix (all but the last row and column of tiles): the scalars of a
+    // lane's rows come from LDS as vectors, all reads in flight together, and the 16 x MT stores per
+    // lane follow each other without a branch or a wait in between.  (Row by row, with two dependent
+    // LDS reads and three branches per row, this took 8,000-11,500 cycles per workgroup, most of it
+    // latency; while a workgroup is in its epilogue its CU has one stream of MFMAs instead of two, and
+    // the kernel's last epilogues are not overlapped with anything.)
+    if (vec_ok && m0 + TM <= M && n0 + BN <= N) {
+        v4f sc[MT][4];
+        v4i rsv[MT][4];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int lrow = wm * (32 * MT) + mt * 32 + 8 * g4 + 4 * (lane >> 5);  // rows lrow .. lrow + 3
+                sc[mt][g4] = *reinterpret_cast<const v4f *>(&s_scale[lrow]);
+                rsv[mt][g4] = *reinterpret_cast<const v4i *>(&s_rowsum[lrow]);
+            }
+        float *orow = out + (size_t)(m0 + wm * (32 * MT) + 4 * (lane >> 5)) * N + col0;
+        int32_t *arow = acc_out ? acc_out + (size_t)(m0 + wm * (32 * MT) + 4 * (lane >> 5)) * N + col0 : nullptr;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int rs = rsv[mt][r >> 2][r & 3];
+                const float as = sc[mt][r >> 2][r & 3];
+                int t[4];
+                float v[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    t[j] = acc[mt][j][r] - rs;
+                    const float f = (float)t[j] * as;  // kernels.rs:168, left to right
+                    v[j] = f * w_scale;
+                }
+                const size_t o = (size_t)(mt * 32 + 8 * (r >> 2) + (r & 3)) * N;
+                __builtin_nontemporal_store(v4f{v[0], v[1], v[2], v[3]}, reinterpret_cast<v4f *>(orow + o));
+                if (arow) __builtin_nontemporal_store(v4i{t[0], t[1], t[2], t[3]}, reinterpret_cast<v4i *>(arow + o));
+            }
+        return;
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll

@@ -12,8 +12,12 @@
 //    issued while step it is multiplied, so HBM latency (each weight byte is used by only
 //    two row tiles per XCD and therefore misses L2) is covered by two K steps.  The loads
 //    are issued from inline assembly, so the compiler neither tracks nor waits for them;
-//    the ring is synchronised by hand: s_waitcnt vmcnt(6) leaves exactly the newest
-//    stage's six loads in flight, then a bare s_barrier.  The ring's three positions are
+//    the ring is synchronised by hand: an s_waitcnt vmcnt(n) that leaves exactly the newest
+//    stage's loads in flight, then a bare s_barrier.  A wave issues such a load in about
+//    33 cycles, in which it issues nothing else: the six loads of a stage are therefore
+//    issued one at a time, each right behind an MFMA that keeps the matrix pipe busy for
+//    32 cycles, and not as a block at the start of the K step (where they held the pipe
+//    idle for 200 of a K step's 1,420 cycles).  The ring's three positions are
 //    written out in the loop body, so LDS addresses are lane constants plus immediates.
 //  * A lane of such a load picks its own global address (a workgroup-uniform base in scalar
 //    registers plus a 32-bit lane offset) but lands at LDS base + 16 * lane,
@@ -89,6 +93,8 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
     constexpr int kAUnits = TM * 8;              // 16-byte units of one activation stage
     constexpr int kLoads = 2 * MT + 2;           // LDS loads per wave and stage
     constexpr int kWaitStage = 0x0070 | kLoads;  // s_waitcnt vmcnt(kLoads) lgkmcnt(0)
+    // at the hand-over inside a K step: the sixth load of a stage is issued behind it (MT = 2)
+    constexpr int kWaitMid = 0x0070 | (MT == 2 ? 5 : 4);
     __shared__ __attribute__((aligned(16))) uint4 smem[3 * (kAUnits + kBUnits)];
     __shared__ __attribute__((aligned(16))) float s_scale[TM];
     __shared__ __attribute__((aligned(16))) int s_rowsum[TM];
@@ -180,6 +186,19 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
         for (int j = 0; j < 2; ++j) dma16(bb, b_lane[j], sb + (4 * j + wave) * 1024);
     };
 
+    // load d of a stage on its own: d < 2 * MT is activation load d, the others are the weight loads
+    auto issue_one = [&](int it, int stage, int d) {
+        const int kk = min(it, iters - 1);
+        if (d < 2 * MT) {
+            const uint32_t sa = lds0 + (uint32_t)(3 * kBUnits + stage * kAUnits) * 16;
+            dma16(a_base + (size_t)kk * BK, a_lane[d], sa + (4 * d + wave) * 1024);
+        } else {
+            const int j = d - 2 * MT;
+            const uint32_t sb = lds0 + (uint32_t)(stage * kBUnits) * 16;
+            dma16(b_base + (size_t)kk * (BK / 16), b_lane[j], sb + (4 * j + wave) * 1024);
+        }
+    };
+
     // fragment addresses (in 16-byte units, relative to a stage)
     const int frow0 = wm * (32 * MT) + (lane & 31), khalf = lane >> 5;
     const int fquad = wn * 32 + (lane & 31);
@@ -223,25 +242,47 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
         bf_n[2] = decode_b(rb[ks].z);
         bf_n[3] = decode_b(rb[ks].w);
     };
-    // sub-step ks: read (read_stage, read_ks), decode dec_ks, multiply ks
-    auto substep = [&](int ks, int read_stage, int read_ks, int dec_ks) {
+    // sub-step ks: read (read_stage, read_ks), decode dec_ks, multiply ks; `mid` runs between the
+    // two halves of the sub-step (a transfer is issued there, behind an MFMA that keeps the pipe busy)
+    auto substep = [&](int ks, int read_stage, int read_ks, int dec_ks, auto mid) {
         lds_reads(read_stage, read_ks);
-        decode_next(dec_ks);
+        bf_n[0] = decode_b(rb[dec_ks].x);
+        bf_n[1] = decode_b(rb[dec_ks].y);
         const v4i af0 = {(int)ra0[ks].x, (int)ra0[ks].y, (int)ra0[ks].z, (int)ra0[ks].w};
         const v4i af1 = {(int)ra1[ks].x, (int)ra1[ks].y, (int)ra1[ks].z, (int)ra1[ks].w};
+        if constexpr (MT == 2) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-            acc[0][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af0, bf[j], acc[0][j], 0, 0, 0);
+            for (int j = 0; j < 4; ++j)
+                acc[0][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af0, bf[j], acc[0][j], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                acc[0][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af0, bf[j], acc[0][j], 0, 0, 0);
+        }
+#pragma unroll
+        for (int g = 0; g < 2 * MT; ++g) {
+            if (g < MT + 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // MFMA
+            __builtin_amdgcn_sched_group_barrier(0x002, 8 / MT, 0);             // VALU
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mid();
+        __builtin_amdgcn_sched_barrier(0);
+        bf_n[2] = decode_b(rb[dec_ks].z);
+        bf_n[3] = decode_b(rb[dec_ks].w);
         if constexpr (MT == 2) {
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 acc[1][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af1, bf[j], acc[1][j], 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int j = 2; j < 4; ++j)
+                acc[0][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af0, bf[j], acc[0][j], 0, 0, 0);
         }
 #pragma unroll
-        for (int g = 0; g < 4 * MT; ++g) {
-            if (g < MT + 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // MFMA
-            __builtin_amdgcn_sched_group_barrier(0x002, 8 / MT, 0);             // VALU
+        for (int g = 0; g < 2 * MT; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);       // MFMA
+            __builtin_amdgcn_sched_group_barrier(0x002, 8 / MT, 0);  // VALU
         }
 #pragma unroll
         for (int j = 0; j < 4; ++j) bf[j] = bf_n[j];
@@ -272,26 +313,33 @@ __global__ __launch_bounds__(kThreads, MT == 2 ? 2 : 3) void gemm_t2_i8_mfma_ker
     for (int j = 0; j < 4; ++j) bf[j] = bf_n[j];
     __builtin_amdgcn_sched_barrier(0);
 
-    // K step `it` on stage cur: start the loads of step it+2 into `fill` - the stage read
+    // K step `it` on stage cur: the loads of step it+2 go into `fill` - the stage read
     // in step it-1, which every wave has left: all its reads were waited for before the
-    // barrier inside step it-1.  After sub-step 1, wait until only those newest kLoads loads
-    // are outstanding (stage nxt has landed) and until this wave's reads of `cur` have
-    // returned, meet, and go on with the reads of nxt.  In the last step nxt holds no
-    // new data; what is read from it is never used.
+    // barrier inside step it-1.  They are issued one by one: before, in the middle of and
+    // behind sub-steps 0 and 1, and (the sixth, MT = 2) in the middle of sub-step 2.  After
+    // sub-step 1, wait until only the newest five (MT = 1: four) loads are outstanding - the
+    // sixth load of stage nxt, issued in step it-1, is older than those, so stage nxt has
+    // landed - and until this wave's reads of `cur` have returned, meet, and go on with the
+    // reads of nxt.  In the last step nxt holds no new data; what is read from it is never used.
     // The loop body is written out for the three positions of the ring, so every LDS
     // address is a lane constant plus an immediate.
     auto kstep = [&](auto cur_tag, int it) {
         constexpr int cur = decltype(cur_tag)::value;
         constexpr int nxt = (cur + 1) % 3, fill = (cur + 2) % 3;
-        issue(it + 2, fill);
+        auto none = [] {};
+        issue_one(it + 2, fill, 0);
         __builtin_amdgcn_sched_barrier(0);
-        substep(0, cur, 2, 1);
-        substep(1, cur, 3, 2);
-        __builtin_amdgcn_s_waitcnt(kWaitStage);
+        substep(0, cur, 2, 1, [&] { issue_one(it + 2, fill, 1); });
+        issue_one(it + 2, fill, 2);
+        __builtin_amdgcn_sched_barrier(0);
+        substep(1, cur, 3, 2, [&] { issue_one(it + 2, fill, 3); });
+        if constexpr (MT == 2) issue_one(it + 2, fill, 4);
+        __builtin_amdgcn_s_waitcnt(kWaitMid);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        substep(2, nxt, 0, 3);
-        substep(3, nxt, 1, 0);
+        if constexpr (MT == 2) substep(2, nxt, 0, 3, [&] { issue_one(it + 2, fill, 5); });
+        else substep(2, nxt, 0, 3, none);
+        substep(3, nxt, 1, 0, none);
     };
     // The K loop runs at a higher wave priority than the epilogue: by default the older workgroup of a
     // CU wins the issue slots, also while it is in its epilogue (conversions, multiplies and stores),

@@ -251,6 +251,68 @@ def test_prefill_tile_model(M, K, N, bm, bn):
     assert (result[:rows, :cols] - rowsum == want).all()
 
 
+def prefill_ring_schedule(mt, iters):
+    """A wave's program of ring events for `iters` K steps, in program order, as gemm_t2_i8_mfma_kernel<mt>
+    issues them: ("load", step, d) starts transfer d of K step `step` into buffer step % 3, ("read", step)
+    reads fragments of that step's buffer, ("wait", n) is s_waitcnt vmcnt(n) lgkmcnt(0), ("barrier",)."""
+    loads = 2 * mt + 2
+    ev = [("load", 0, d) for d in range(loads)] + [("load", 1, d) for d in range(loads)]
+    ev += [("wait", loads), ("barrier",), ("read", 0), ("read", 0)]
+    for it in range(iters):
+        ev += [("load", it + 2, 0), ("read", it), ("load", it + 2, 1)]           # sub-step 0 and its middle
+        ev += [("load", it + 2, 2), ("read", it), ("load", it + 2, 3)]           # sub-step 1
+        if mt == 2:
+            ev += [("load", it + 2, 4)]
+        ev += [("wait", 5 if mt == 2 else 4), ("barrier",)]
+        ev += [("read", it + 1)]                                                   # sub-step 2
+        if mt == 2:
+            ev += [("load", it + 2, 5)]
+        ev += [("read", it + 1)]                                                   # sub-step 3
+    ev += [("wait", 0)]
+    return ev, loads
+
+
+@pytest.mark.parametrize("mt,iters", [(2, 1), (2, 2), (2, 7), (1, 1), (1, 5)])
+def test_prefill_ring_schedule_never_reads_early_or_overwrites_late(mt, iters):
+    """The hand-counted vmcnt of the prefill kernel's three-stage ring, replayed: loads retire in order,
+    a wait for n leaves the newest n in flight, and every wave runs the same program between barriers.
+    (a) Every read finds all loads of its K step landed in every wave: each wave waited for them before
+    the last barrier.  (b) A load into a buffer is issued only behind a barrier that every wave reached
+    after its last read of that buffer's previous content had returned."""
+    ev, loads = prefill_ring_schedule(mt, iters)
+    in_flight = []                 # (step, d), oldest first
+    landed = set()                 # loads this wave knows to have landed
+    published = set()              # landed before the last barrier: true of all four waves
+    reads_returned = set()         # steps whose reads so far have returned (lgkmcnt(0)), as of the last wait
+    reads_issued = []              # steps read since the last wait
+    safe_to_overwrite = set()      # steps every wave has finished reading, as of the last barrier
+    last_read_at = {}
+    for i, e in enumerate(ev):
+        if e[0] == "read":
+            last_read_at[e[1]] = i
+    for i, e in enumerate(ev):
+        if e[0] == "load":
+            step = e[1]
+            if step >= 3:
+                assert step - 3 in safe_to_overwrite, (i, e)
+            in_flight.append((step, e[2]))
+        elif e[0] == "wait":
+            while len(in_flight) > e[1]:
+                landed.add(in_flight.pop(0))
+            reads_returned = set(reads_issued)
+            pending_done = {s for s in reads_returned if last_read_at[s] < i}
+            reads_done_before_wait = pending_done
+        elif e[0] == "barrier":
+            published = set(landed)
+            safe_to_overwrite |= reads_done_before_wait
+        elif e[0] == "read":
+            step = e[1]
+            if step < iters:       # past the last step the buffer holds nothing new and the result is unused
+                assert all((step, d) in published for d in range(loads)), (i, e)
+            reads_issued.append(step)
+    assert not in_flight           # nothing still writes LDS when the epilogue reuses it
+
+
 # ---- decode GEMV (gemv.hip): the 4-bit planes that feed v_dot8 ---------------------------------------------
 
 def test_gemv_nibble_planes_reproduce_the_int8_dot_product():

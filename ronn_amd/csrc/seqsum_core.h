@@ -144,6 +144,36 @@ SEQ_HD SeqMap seq_append_abs(SeqMap m, float a, uint32_t es, float scale) {
     return m;
 }
 
+// The map of sixteen consecutive terms a[0..15] (non-negative; a term of +0.0 is the identity and
+// stands for an element that the mask skips) for a state of exponent es, scale = seq_ulp_scale(es).
+// A term changes k by q + [r > u/2] = round-to-nearest(v), v = a * scale, whatever k is - unless v
+// lies exactly half way between two integers, the one case in which the parity of k decides.  So
+// when none of the sixteen is such a tie (the rule: a tie needs a term whose low bits are exactly
+// 1000...0 at the state's ulp), the map is one sum of sixteen independent roundings, d0 = d1, and
+// the sixteen terms do not wait for each other as they do in seq_append_abs; with a tie among them
+// the terms are appended one by one.  v is clamped to 2^25 = SEQ_SAT first (NaN included: the
+// minimum of a NaN and a number is the number), so a sum of sixteen stays below 2^32 and a term far
+// above the binade saturates the map exactly as it does in seq_append_abs.
+SEQ_HD SeqMap seq_map16(const float *a, uint32_t es, float scale) {
+    SeqMap m = seq_identity();
+    bool tie = es < 26u;  // below that the term is split in integer arithmetic
+    if (!tie) {
+        uint32_t sum = 0u;
+        for (int i = 0; i < 16; ++i) {
+            const float v = __builtin_fminf(a[i] * scale, 33554432.0f);
+            const float r = __builtin_rintf(v);  // to nearest, ties to even (the default rounding mode)
+            tie = tie || __builtin_fabsf(v - r) == 0.5f;
+            sum += (uint32_t)r;
+        }
+        m.d0 = m.d1 = seq_min_u32(sum, SEQ_SAT);
+    }
+    if (tie) {
+        m = seq_identity();
+        for (int i = 0; i < 16; ++i) m = seq_append_abs(m, a[i], es, scale);
+    }
+    return m;
+}
+
 // Map of "first a, then b".
 SEQ_HD SeqMap seq_compose(SeqMap a, SeqMap b) {
     SeqMap r;
@@ -177,6 +207,52 @@ SEQ_HD uint64_t seq_next_window(uint64_t pos, uint64_t total_blocks, double s_no
     if (win < 64u) win = 64u;
     if (win > total_blocks - pos) win = total_blocks - pos;
     return win;
+}
+
+// ---- windows that span several binades ------------------------------------------------------
+// The first binades are short: S of similar terms doubles when the position doubles, so the
+// first 8192 blocks hold thirteen of them, and a window per binade spends its time on launches.
+// A window that starts below SEQ_MULTI_LIMIT therefore carries TWO maps per block, for the
+// exponents e and e + 1 where e = seq_multi_es_lo() is the exponent that a cautious prediction
+// of S gives for that block: L(i) = S0 + i * rate_lo with rate_lo = 0.9 x the growth per block
+// measured over the previous window.  The true S entering block i has exponent e or e + 1
+// whenever L(i) <= S < 2 L(i), i.e. for any growth between 0.9 and 1.8 times the measured one;
+// the scan then walks through the binades inside one window (scan to the crossing, replay that
+// block, go on with the other map) and ends the window early at the first block whose pair does
+// not hold the exponent S really has.  Block 0 of a window always does (L(0) = S0).
+#define SEQ_MULTI_LIMIT 8192u
+
+SEQ_HD uint32_t seq_multi_es_lo(uint32_t s0_bits, uint32_t rate_lo_bits, uint32_t i) {
+    float s0, r;
+    __builtin_memcpy(&s0, &s0_bits, 4);
+    __builtin_memcpy(&r, &rate_lo_bits, 4);
+    const float l = __builtin_fmaf((float)i, r, s0);  // one rounding, the same wherever it is evaluated
+    uint32_t b;
+    __builtin_memcpy(&b, &l, 4);
+    const uint32_t e = (b >> 23) & 0xffu;
+    return e == 0u ? 1u : (e > 254u ? 254u : e);
+}
+
+// rate_lo as f32 bits from the growth per block of the last window (0 when there is none to trust)
+SEQ_HD uint32_t seq_multi_rate_lo(double rate) {
+    float r = 0.0f;
+    if (rate > 0.0 && rate < 1e38) r = (float)(0.9 * rate);
+    uint32_t b;
+    __builtin_memcpy(&b, &r, 4);
+    return b;
+}
+
+// The next window: its size, and in *multi whether it carries two maps per block.
+SEQ_HD uint64_t seq_plan_window(uint64_t pos, uint64_t total_blocks, double s_now, double rate, uint32_t *multi) {
+    if (pos > 0u && pos < SEQ_MULTI_LIMIT && isfinite(s_now)) {
+        uint64_t win = 255u * pos + 64u;  // the second window already measures the growth over hundreds of blocks
+        if (win > SEQ_MULTI_LIMIT - pos) win = SEQ_MULTI_LIMIT - pos;
+        if (win > total_blocks - pos) win = total_blocks - pos;
+        *multi = 1u;
+        return win;
+    }
+    *multi = 0u;
+    return seq_next_window(pos, total_blocks, s_now, rate);
 }
 
 #endif  // RONN_SEQSUM_CORE_H

@@ -242,8 +242,10 @@ struct SeqState {
     uint32_t done;      // all blocks folded, or S no longer finite: queued kernels just return
     uint32_t error;     // a window made no progress (internal error)
     uint32_t saw_nan;   // set by any_nan_kernel
-    uint32_t pad;
+    uint32_t multi;     // the window carries two maps per block (seq_plan_window)
     uint64_t fresh_from;  // blocks from here on have not been seen by any window yet
+    uint32_t rate_lo;   // multi: the cautious growth of S per block (f32 bits) behind the blocks' exponents
+    uint32_t pad;
 };
 
 // A SeqMap from another lane by a DPP move: lanes without a source (and rows outside the
@@ -256,31 +258,34 @@ __device__ __forceinline__ SeqMap seq_dpp(SeqMap m) {
     return o;
 }
 
-// One SeqMap per block of 4096 elements, valid for a state of biased exponent `es`.
+// One SeqMap per block of 4096 elements, valid for a state of biased exponent `es` - or, in a
+// window that spans several binades (state->multi), two per block: for the exponents e and e + 1,
+// e = seq_multi_es_lo(block), stored side by side (maps[2 * block], maps[2 * block + 1]).
 // The window and the exponent come from the state; the grid strides over the window's blocks.
 // With `packed` given (masked sums only: thr is the ternary threshold) the kernel also packs
 // every block that no earlier window has touched - a thread's 16 elements are one 32-bit word
 // of the reference's layout - and adds their survivors to this workgroup's counter: the
 // scale's sum and the packing then share one pass over the tensor.
-__global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
+template <bool MULTI>
+__device__ __forceinline__ void seq_block_maps_body(
     const float *__restrict__ x, uint64_t n, int use_mask, float thr,
     const SeqState *__restrict__ state, SeqMap *__restrict__ maps, uint32_t *__restrict__ packed,
-    unsigned long long *__restrict__ count_parts) {
-    __shared__ SeqMap s_wave[kBlock / 64];
-    __shared__ unsigned s_cnt[kBlock / 64];
-    if (state->done) return;
+    unsigned long long *__restrict__ count_parts, SeqMap *s_wave, unsigned *s_cnt) {
     const uint32_t win = state->win;
     const uint64_t fresh_from = state->fresh_from, pos = state->pos;
     unsigned fresh_count = 0;
     const uint64_t first = state->pos * kSeqTile;
-    uint32_t es, k_unused;
-    seq_state_split(state->s_bits, &es, &k_unused);
-    const float scale = seq_ulp_scale(es < 26u ? 26u : es);
+    const uint32_t s_bits = state->s_bits, rate_lo = state->rate_lo;
+    uint32_t es0, k_unused;
+    seq_state_split(s_bits, &es0, &k_unused);
   for (uint32_t blk = blockIdx.x; blk < win; blk += gridDim.x) {
+    const uint32_t es = MULTI ? seq_multi_es_lo(s_bits, rate_lo, blk) : es0;
+    const float scale = seq_ulp_scale(es < 26u ? 26u : es);
+    const float scale_b = seq_ulp_scale(es + 1u < 26u ? 26u : es + 1u);
     uint64_t base = first + (uint64_t)blk * kSeqTile + (uint64_t)threadIdx.x * 16;
-    SeqMap m = seq_identity();
     const bool fresh = packed != nullptr && pos + blk >= fresh_from;
     uint32_t word = 0;
+    float am[16];  // |x| of the elements that count, +0.0 (the identity as a term) for the others
     if (base + 16 <= n) {
         float4 v[4];
 #pragma unroll
@@ -292,7 +297,7 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
             for (int i = 0; i < 4; ++i) {
                 float a = fabsf(e[i]);
                 bool take = use_mask ? (a > thr) : true;
-                if (take) m = seq_append_abs(m, a, es, scale);
+                am[4 * j + i] = take ? a : 0.0f;
                 if (fresh) {
                     word |= ternary_code(e[i], thr) << (2 * (4 * j + i));
                     fresh_count += take ? 1u : 0u;
@@ -301,13 +306,15 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
         }
         if (fresh) packed[base >> 4] = word;
     } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) am[i] = 0.0f;
         for (int i = 0; i < 16; ++i) {
             uint64_t idx = base + i;
             if (idx < n) {
                 float e = x[idx];
                 float a = fabsf(e);
                 bool take = use_mask ? (a > thr) : true;
-                if (take) m = seq_append_abs(m, a, es, scale);
+                am[i] = take ? a : 0.0f;
                 if (fresh) {
                     word |= ternary_code(e, thr) << (2 * i);
                     fresh_count += take ? 1u : 0u;
@@ -316,20 +323,37 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
         }
         if (fresh && base < n) packed[base >> 4] = word;  // tail bits stay zero
     }
+    SeqMap m = seq_map16(am, es, scale), mb = seq_identity();
+    if (MULTI) mb = seq_map16(am, es + 1u, scale_b);
     // ordered reduction of the wave by DPP moves (each lane absorbs what lies to its left):
     // lane 63 ends up with the map of all 1024 elements
-    m = seq_compose(seq_dpp<0x111, 0xf>(m), m);  // row_shr:1
-    m = seq_compose(seq_dpp<0x112, 0xf>(m), m);  // row_shr:2
-    m = seq_compose(seq_dpp<0x114, 0xf>(m), m);  // row_shr:4
-    m = seq_compose(seq_dpp<0x118, 0xf>(m), m);  // row_shr:8
-    m = seq_compose(seq_dpp<0x142, 0xa>(m), m);  // row_bcast15
-    m = seq_compose(seq_dpp<0x143, 0xc>(m), m);  // row_bcast31
-    if ((threadIdx.x & 63) == 63) s_wave[threadIdx.x >> 6] = m;
+    auto wave_fold = [](SeqMap v) {
+        v = seq_compose(seq_dpp<0x111, 0xf>(v), v);  // row_shr:1
+        v = seq_compose(seq_dpp<0x112, 0xf>(v), v);  // row_shr:2
+        v = seq_compose(seq_dpp<0x114, 0xf>(v), v);  // row_shr:4
+        v = seq_compose(seq_dpp<0x118, 0xf>(v), v);  // row_shr:8
+        v = seq_compose(seq_dpp<0x142, 0xa>(v), v);  // row_bcast15
+        v = seq_compose(seq_dpp<0x143, 0xc>(v), v);  // row_bcast31
+        return v;
+    };
+    m = wave_fold(m);
+    if (MULTI) mb = wave_fold(mb);
+    constexpr int NW = kBlock / 64;
+    if ((threadIdx.x & 63) == 63) {
+        s_wave[threadIdx.x >> 6] = m;
+        if (MULTI) s_wave[NW + (threadIdx.x >> 6)] = mb;
+    }
     __syncthreads();
     if (threadIdx.x == 0) {
         SeqMap t = s_wave[0];
-        for (int w = 1; w < kBlock / 64; ++w) t = seq_compose(t, s_wave[w]);
-        maps[blk] = t;
+        for (int w = 1; w < NW; ++w) t = seq_compose(t, s_wave[w]);
+        if (MULTI) {
+            SeqMap u = s_wave[NW];
+            for (int w = 1; w < NW; ++w) u = seq_compose(u, s_wave[NW + w]);
+            reinterpret_cast<uint4 *>(maps)[blk] = make_uint4(t.d0, t.d1, u.d0, u.d1);
+        } else {
+            maps[blk] = t;
+        }
     }
     __syncthreads();  // s_wave is rewritten in the next turn
   }
@@ -345,6 +369,19 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
             if (t) count_parts[blockIdx.x] += t;
         }
     }
+}
+
+__global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
+    const float *__restrict__ x, uint64_t n, int use_mask, float thr,
+    const SeqState *__restrict__ state, SeqMap *__restrict__ maps, uint32_t *__restrict__ packed,
+    unsigned long long *__restrict__ count_parts) {
+    __shared__ SeqMap s_wave[2 * (kBlock / 64)];
+    __shared__ unsigned s_cnt[kBlock / 64];
+    if (state->done) return;
+    if (state->multi)
+        seq_block_maps_body<true>(x, n, use_mask, thr, state, maps, packed, count_parts, s_wave, s_cnt);
+    else
+        seq_block_maps_body<false>(x, n, use_mask, thr, state, maps, packed, count_parts, s_wave, s_cnt);
 }
 
 __global__ __launch_bounds__(kBlock) void fill_u64_kernel(unsigned long long *p, int n) {
@@ -391,15 +428,151 @@ __device__ __forceinline__ SeqMap seq_block_before(SeqMap m, SeqMap *s_w, SeqMap
     if (lane == 63 && wave < NW) s_w[wave] = m;
     const SeqMap ex = seq_dpp<0x138, 0xf>(m);  // wave_shr:1: exclusive inside the wave, lane 0 reads the identity
     __syncthreads();
-    SeqMap pre = seq_identity(), tot = seq_identity();
-#pragma unroll
-    for (int w = 0; w < NW; ++w) {
-        const SeqMap sw = s_w[w];
-        if (w < wave) pre = seq_compose(pre, sw);
-        tot = seq_compose(tot, sw);
+    // the waves' totals, one per lane of the first row, scanned the same way (four steps instead
+    // of a chain of NW compositions); lane w - 1 then holds everything before wave w
+    static_assert(NW <= 16, "the waves' totals must fit one row of lanes");
+    SeqMap v = seq_identity();
+    if (lane < NW) v = s_w[lane];
+    v = seq_compose(seq_dpp<0x111, 0xf>(v), v);  // row_shr:1
+    v = seq_compose(seq_dpp<0x112, 0xf>(v), v);  // row_shr:2
+    if (NW > 4) v = seq_compose(seq_dpp<0x114, 0xf>(v), v);  // row_shr:4
+    if (NW > 8) v = seq_compose(seq_dpp<0x118, 0xf>(v), v);  // row_shr:8
+    const int w_uni = __builtin_amdgcn_readfirstlane(wave);
+    SeqMap pre = seq_identity(), tot;
+    tot.d0 = (uint32_t)__builtin_amdgcn_readlane((int)v.d0, NW - 1);
+    tot.d1 = (uint32_t)__builtin_amdgcn_readlane((int)v.d1, NW - 1);
+    if (w_uni > 0) {
+        pre.d0 = (uint32_t)__builtin_amdgcn_readlane((int)v.d0, w_uni - 1);
+        pre.d1 = (uint32_t)__builtin_amdgcn_readlane((int)v.d1, w_uni - 1);
     }
     *total = tot;
     return seq_compose(pre, ex);
+}
+
+// Resolves one block of 4096 elements from the state (es, k_cur) that enters it, called by all
+// 1024 threads of the window-end kernel.  The block's 256 chunks of 16 elements are mapped
+// (threads 0..255, one chunk each) and scanned from the entering state; the one chunk in which
+// k reaches 2^24 is replayed with ordinary f32 additions, which moves S into a new binade; the
+// chunks after it are mapped again for that binade, and so on to the end of the block.  Early
+// blocks cross several binades (S doubles every few elements at first), later ones at most one.
+// Only the first four waves work: the other twelve share their SIMDs, and every instruction
+// they issue delays the four (a turn of the loop took 5,300 cycles with all sixteen running the
+// same code), so they only keep the barriers and read the loop's conditions from LDS.
+// Returns the state after the block as f32 bits (possibly +Inf or NaN) - in the first four waves;
+// the same value is left in *s_bits_now for the others, who read it behind a barrier of the
+// caller's.  s_w, s_first and s_bits_now are LDS scratch; the caller puts a barrier before it
+// touches them again.
+__device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x, uint64_t n, uint64_t block_base,
+                                                     int use_mask, float thr, uint32_t es, uint32_t k_cur,
+                                                     SeqMap *s_w, unsigned *s_first, uint32_t *s_bits_now) {
+    const uint32_t t = threadIdx.x;
+    constexpr int NW = kBlock / 64;
+    const bool worker = __builtin_amdgcn_readfirstlane((int)(t >> 6)) < NW;  // wave-uniform
+    if (!worker) {
+        // the barriers of the loop below, in the same order, and its exits
+        for (int guard = 0; guard <= kBlock; ++guard) {
+            __syncthreads();  // (1) wave totals written
+            __syncthreads();  // (2) crossing chunk known
+            const uint32_t tstar = *s_first;
+            if (tstar == 0xffffffffu) break;
+            __syncthreads();  // (3) chunk replayed
+            const uint32_t bits = *s_bits_now;
+            if (((bits >> 23) & 0xffu) == 0xffu) {
+                __syncthreads();  // (4) NaN behind an Inf
+                break;
+            }
+            if (tstar + 1u >= (uint32_t)kBlock) break;
+        }
+        return 0u;
+    }
+    const uint64_t base = block_base + (uint64_t)t * 16;
+    float a[16];
+    if (base + 16 <= n && (reinterpret_cast<uintptr_t>(x + base) & 15u) == 0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float4 v = reinterpret_cast<const float4 *>(x + base)[j];
+            a[4 * j] = fabsf(v.x), a[4 * j + 1] = fabsf(v.y), a[4 * j + 2] = fabsf(v.z), a[4 * j + 3] = fabsf(v.w);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) a[i] = 0.0f;
+        for (int i = 0; i < 16; ++i) {
+            const uint64_t idx = base + i;
+            if (idx < n) a[i] = fabsf(x[idx]);
+        }
+    }
+    // a skipped element adds +0.0, which leaves any S >= 0 (and NaN/Inf) unchanged, and as a
+    // term of a map it is the identity
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a[i] = (!use_mask || a[i] > thr) ? a[i] : 0.0f;
+    const int lane = t & 63, wave = t >> 6;
+    uint32_t done = 0;  // chunks [0, done) are already folded into (es, k_cur)
+    uint32_t result_bits = 0;
+    for (int guard = 0; guard <= kBlock; ++guard) {
+        SeqMap m = seq_identity();
+        if (t >= done) m = seq_map16(a, es, seq_ulp_scale(es < 26u ? 26u : es));
+        if (t == 0) *s_first = 0xffffffffu;
+        // inclusive scan of the wave, the waves' totals through LDS
+        SeqMap inc = m;
+        inc = seq_compose(seq_dpp<0x111, 0xf>(inc), inc);  // row_shr:1
+        inc = seq_compose(seq_dpp<0x112, 0xf>(inc), inc);  // row_shr:2
+        inc = seq_compose(seq_dpp<0x114, 0xf>(inc), inc);  // row_shr:4
+        inc = seq_compose(seq_dpp<0x118, 0xf>(inc), inc);  // row_shr:8
+        inc = seq_compose(seq_dpp<0x142, 0xa>(inc), inc);  // row_bcast15
+        inc = seq_compose(seq_dpp<0x143, 0xc>(inc), inc);  // row_bcast31
+        if (lane == 63) s_w[wave] = inc;
+        const SeqMap ex = seq_dpp<0x138, 0xf>(inc);  // wave_shr:1: exclusive inside the wave
+        __syncthreads();  // (1)
+        SeqMap pre = seq_identity(), all = seq_identity();
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const SeqMap sw = s_w[w];
+            if (w < wave) pre = seq_compose(pre, sw);
+            all = seq_compose(all, sw);
+        }
+        const SeqMap before = seq_compose(pre, ex);
+        const uint32_t k = seq_apply(before, k_cur);
+        const bool crosses = t >= done && k < SEQ_K_LIMIT && seq_apply(m, k) >= SEQ_K_LIMIT;
+        if (crosses) atomicMin(s_first, t);
+        const uint32_t k_end = seq_apply(all, k_cur);  // state after the block if no crossing
+        __syncthreads();  // (2)
+        const uint32_t tstar = *s_first;
+        if (tstar == 0xffffffffu) {
+            result_bits = seq_state_join(es, k_end);
+            break;
+        }
+        if (t == tstar) {
+            float sum = __uint_as_float(seq_state_join(es, k));
+#pragma unroll
+            for (int i = 0; i < 16; ++i) sum = sum + a[i];
+            *s_bits_now = __float_as_uint(sum);
+        }
+        __syncthreads();  // (3)
+        result_bits = *s_bits_now;
+        done = tstar + 1;
+        if (((result_bits >> 23) & 0xffu) == 0xffu) {
+            // S is +Inf or NaN.  +Inf turns into NaN if a NaN follows inside this block.
+            bool nan_after = false;
+            if (t >= done) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) nan_after |= (a[i] != a[i]);
+            }
+            if (nan_after) atomicOr(s_bits_now, 0x7fc00000u);  // Inf | quiet bit = NaN
+            __syncthreads();  // (4)
+            result_bits = *s_bits_now;
+            break;
+        }
+        if (done >= (uint32_t)kBlock) break;
+        seq_state_split(result_bits, &es, &k_cur);
+        // (no barrier here: s_first was last read before barrier (3), s_w before (2), and
+        // s_bits_now is written again only behind the next turn's barrier (2))
+    }
+    // For the waves that only kept the barriers the result is left in LDS (the caller puts a
+    // barrier before reading it).  The store cannot overtake a read: with no crossing in this turn
+    // nobody has read s_bits_now since the last turn's barrier (3), two barriers ago; on the other
+    // exits it holds this very value already.
+    if (t == 0) *s_bits_now = result_bits;
+    return result_bits;
 }
 
 // One workgroup of 1024 threads ends a window.
@@ -411,16 +584,22 @@ __device__ __forceinline__ SeqMap seq_block_before(SeqMap m, SeqMap *s_w, SeqMap
 //     new binade; the chunks after it are mapped again for that binade, and so on to the
 //     end of the block.  Early blocks cross several binades (S doubles every few elements
 //     at first), later ones at most one.
+// A window with two maps per block (state->multi) repeats (1) and (2): after the replay S is in a
+// new binade, for which the blocks that follow carry their other map, and so on until the window
+// ends or a block's pair does not hold the exponent S has.
 // The new state goes to device memory (for the next window's kernels) and to the pinned
 // host mailbox (the host reads it after synchronising: it sizes the next window).
 __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     const SeqMap *__restrict__ maps, const float *__restrict__ x, uint64_t n, uint64_t total_blocks,
     int use_mask, float thr, SeqState *__restrict__ state, SeqState *__restrict__ host_copy,
     int mirror /* the last launch of a batch: the host reads the state after it */) {
+    extern __shared__ uint4 s_maps[];  // SEQ_MULTI_LIMIT units: the maps of a window with two per block
     __shared__ SeqMap s_w[16];
     __shared__ unsigned s_first;
     __shared__ uint32_t s_cross_block, s_cross_k;
     __shared__ uint32_t s_bits_now;
+    __shared__ unsigned long long s_min64;
+    __shared__ uint32_t s_edge[64];
     const uint32_t t = threadIdx.x;
     // Windows of up to 1024 blocks (most of them) have one map per thread: it is requested
     // here, before the state is known, so that the two round trips overlap (the buffer holds
@@ -451,7 +630,10 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         next.pos = pos;
         next.error = (advanced == 0 || advanced > nblocks) ? 1u : 0u;
         next.done = (pos >= total_blocks || !finite || next.error) ? 1u : 0u;
-        next.win = next.done ? 0u : (uint32_t)seq_next_window(pos, total_blocks, s_after, rate);
+        uint32_t next_multi = 0u;
+        next.win = next.done ? 0u : (uint32_t)seq_plan_window(pos, total_blocks, s_after, rate, &next_multi);
+        next.multi = next.done ? 0u : next_multi;
+        next.rate_lo = seq_multi_rate_lo(rate);
         next.saw_nan = 0;
         next.pad = 0;
         const uint64_t seen = pos0 + nblocks, before = state->fresh_from;
@@ -459,6 +641,110 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         *state = next;
         if (mirror) *host_copy = next;  // a store to pinned host memory: only when somebody will look
     };
+
+    // ---- a window with two maps per block: through as many binades as the maps hold ---------
+    if (state->multi) {
+        // at most SEQ_MULTI_LIMIT blocks: eight per thread, loaded once (both maps of a block are
+        // one 16-byte load)
+        const uint32_t rate_lo = state->rate_lo;
+        if (nblocks > SEQ_MULTI_LIMIT) {  // not a window the plan makes: reported as an internal error
+            if (t == 0) finish(bits0, 0);
+            return;
+        }
+        // The window's maps go to LDS once (both maps of a block are one 16-byte unit): kept in
+        // registers across the replays they did not fit and were spilled.
+        for (uint32_t b = t; b < nblocks; b += 1024u) s_maps[b] = reinterpret_cast<const uint4 *>(maps)[b];
+        __syncthreads();
+        // s_edge[i]: the first block of the window whose lower exponent exceeds es0 + i (nblocks if
+        // there is none).  The exponents never fall along the window, so this is the first b with
+        // S0 + b * rate_lo >= 2^(e+1-127): guessed by a division, settled with the predicate itself.
+        constexpr uint32_t kEdges = 64;
+        const uint32_t es0 = es;
+        if (t < kEdges) {
+            const uint32_t e = es0 + t, a = 0u, z = nblocks;
+            const float s0 = __uint_as_float(bits0), r = __uint_as_float(rate_lo);
+            uint32_t g = a;
+            if (e + 1u <= 254u && r > 0.0f) {
+                const float edge = __uint_as_float((e + 1u) << 23);
+                const float q = (edge - s0) / r;
+                g = q <= (float)a ? a : (q >= (float)z ? z : (uint32_t)q);
+            }
+            int steps = 0;
+            while (g > a && seq_multi_es_lo(bits0, rate_lo, g - 1u) > e && steps < 8) --g, ++steps;
+            while (g < z && !(seq_multi_es_lo(bits0, rate_lo, g) > e) && steps < 16) ++g, ++steps;
+            const bool settled = (g == a || !(seq_multi_es_lo(bits0, rate_lo, g - 1u) > e)) &&
+                                 (g == z || seq_multi_es_lo(bits0, rate_lo, g) > e);
+            if (!settled) {  // the guess was far off (a rate next to nothing): bisect
+                uint32_t lo2 = a, hi2 = z;
+                while (lo2 < hi2) {
+                    const uint32_t mid = lo2 + ((hi2 - lo2) >> 1);
+                    if (seq_multi_es_lo(bits0, rate_lo, mid) > e) hi2 = mid; else lo2 = mid + 1u;
+                }
+                g = lo2;
+            }
+            s_edge[t] = g;
+        }
+        __syncthreads();
+        uint32_t b_cur = 0, cur_bits = bits0;
+        for (int guard = 0; guard < 48; ++guard) {
+            uint32_t k_in;
+            seq_state_split(cur_bits, &es, &k_in);
+            // The blocks from b_cur on whose pair holds `es` reach up to the first one whose lower
+            // exponent exceeds es - provided the pair of b_cur itself is not below es; among them,
+            // those before b_eq stand for es with their second map, the others with their first.
+            if (es - es0 >= kEdges) break;  // further than the table reaches: the next window starts here
+            const uint32_t range_end = s_edge[es - es0];
+            const uint32_t b_eq = es == es0 ? 0u : s_edge[es - es0 - 1u];  // first block whose lower exponent is es
+            // b_cur's pair must hold es: its lower exponent is es (b_cur >= b_eq) or es - 1
+            const uint32_t b_lowest = es - es0 >= 2u ? s_edge[es - es0 - 2u] : 0u;  // first block with es - 1
+            if (b_cur >= range_end || b_cur < b_lowest) break;  // the prediction has lost S
+            // the range in equal shares (at most eight blocks per thread)
+            const uint32_t chunk = (range_end - b_cur + 1023u) / 1024u;
+            const uint32_t lo = b_cur + t * chunk;
+            const uint32_t hi = lo + chunk < range_end ? lo + chunk : range_end;
+            auto pick = [&](uint32_t b) {
+                const uint4 mm = s_maps[b];
+                SeqMap r;
+                r.d0 = b < b_eq ? mm.z : mm.x;
+                r.d1 = b < b_eq ? mm.w : mm.y;
+                return r;
+            };
+            SeqMap mine = seq_identity();
+            for (uint32_t b2 = lo; b2 < hi; ++b2) mine = seq_compose(mine, pick(b2));
+            if (t == 0) s_min64 = ~0ull;
+            SeqMap all;
+            const SeqMap before = seq_block_before<16>(mine, s_w, &all);
+            uint32_t k = seq_apply(before, k_in);
+            if (k < SEQ_K_LIMIT) {
+                for (uint32_t b2 = lo; b2 < hi; ++b2) {
+                    const uint32_t k2 = seq_apply(pick(b2), k);
+                    if (k2 >= SEQ_K_LIMIT) {
+                        // the first crossing block and the k that enters it, as one 64-bit minimum
+                        atomicMin(&s_min64, ((unsigned long long)b2 << 32) | k);
+                        break;
+                    }
+                    k = k2;
+                }
+            }
+            __syncthreads();
+            const unsigned long long first_cross = s_min64;
+            if (first_cross == ~0ull) {
+                // no crossing up to range_end: the state there is what all maps of the range give
+                cur_bits = seq_state_join(es, seq_apply(all, k_in));
+                b_cur = range_end;
+                break;  // the window is through, or the next block's pair does not hold es
+            }
+            const uint32_t cb = (uint32_t)(first_cross >> 32), k_cb = (uint32_t)first_cross;
+            (void)seq_replay_block(x, n, first + (uint64_t)cb * kSeqTile, use_mask, thr, es, k_cb, s_w, &s_first,
+                                   &s_bits_now);
+            __syncthreads();  // the result is in LDS; s_w and s_min64 are rewritten in the next turn
+            cur_bits = s_bits_now;
+            b_cur = cb + 1u;
+            if (((cur_bits >> 23) & 0xffu) == 0xffu || b_cur >= nblocks) break;
+        }
+        if (t == 0) finish(cur_bits, b_cur);
+        return;
+    }
 
     // ---- (1) scan -----------------------------------------------------------------------
     {
@@ -562,89 +848,9 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         return;
     }
 
-    // ---- (2) replay of block cb: threads 0..255 hold a chunk, everybody keeps the barriers
-    const bool holds = t < (uint32_t)kBlock;
-    const uint64_t base = first + (uint64_t)cb * kSeqTile + (uint64_t)t * 16;
-    float a[16];
-    bool take[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        a[i] = 0.0f;
-        take[i] = false;
-    }
-    if (holds) {
-        if (base + 16 <= n && (reinterpret_cast<uintptr_t>(x + base) & 15u) == 0) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float4 v = reinterpret_cast<const float4 *>(x + base)[j];
-                a[4 * j] = fabsf(v.x), a[4 * j + 1] = fabsf(v.y), a[4 * j + 2] = fabsf(v.z), a[4 * j + 3] = fabsf(v.w);
-            }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) take[i] = use_mask ? (a[i] > thr) : true;
-        } else {
-            for (int i = 0; i < 16; ++i) {
-                const uint64_t idx = base + i;
-                if (idx < n) {
-                    a[i] = fabsf(x[idx]);
-                    take[i] = use_mask ? (a[i] > thr) : true;
-                }
-            }
-        }
-        // a skipped element adds +0.0, which leaves any S >= 0 (and NaN/Inf) unchanged
-#pragma unroll
-        for (int i = 0; i < 16; ++i) a[i] = take[i] ? a[i] : 0.0f;
-    }
-    uint32_t done = 0;  // chunks [0, done) are already folded into (es, k_cur)
-    uint32_t result_bits = 0;
-    for (int guard = 0; guard <= kBlock; ++guard) {
-        SeqMap m = seq_identity();
-        if (holds && t >= done) {
-            const float scale = seq_ulp_scale(es < 26u ? 26u : es);
-#pragma unroll
-            for (int i = 0; i < 16; ++i)
-                if (take[i]) m = seq_append_abs(m, a[i], es, scale);
-        }
-        if (t == 0) s_first = 0xffffffffu;
-        SeqMap all;
-        const SeqMap before = seq_block_before<kBlock / 64>(m, s_w, &all);
-        uint32_t k = 0;
-        if (holds) {
-            k = seq_apply(before, k_cur);
-            const bool crosses = t >= done && k < SEQ_K_LIMIT && seq_apply(m, k) >= SEQ_K_LIMIT;
-            if (crosses) atomicMin(&s_first, t);
-        }
-        const uint32_t k_end = seq_apply(all, k_cur);  // state after the block if no crossing
-        __syncthreads();
-        const uint32_t tstar = s_first;
-        if (tstar == 0xffffffffu) {
-            result_bits = seq_state_join(es, k_end);
-            break;
-        }
-        if (t == tstar) {
-            float sum = __uint_as_float(seq_state_join(es, k));
-#pragma unroll
-            for (int i = 0; i < 16; ++i) sum = sum + a[i];
-            s_bits_now = __float_as_uint(sum);
-        }
-        __syncthreads();
-        result_bits = s_bits_now;
-        done = tstar + 1;
-        if (((result_bits >> 23) & 0xffu) == 0xffu) {
-            // S is +Inf or NaN.  +Inf turns into NaN if a NaN follows inside this block.
-            bool nan_after = false;
-            if (holds && t >= done) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i) nan_after |= (a[i] != a[i]);
-            }
-            if (nan_after) atomicOr(&s_bits_now, 0x7fc00000u);  // Inf | quiet bit = NaN
-            __syncthreads();
-            result_bits = s_bits_now;
-            break;
-        }
-        if (done >= (uint32_t)kBlock) break;
-        seq_state_split(result_bits, &es, &k_cur);
-        __syncthreads();  // s_first / s_bits_now are rewritten in the next turn
-    }
+    // ---- (2) replay of block cb
+    const uint32_t result_bits = seq_replay_block(x, n, first + (uint64_t)cb * kSeqTile, use_mask, thr, es, k_cur,
+                                                  s_w, &s_first, &s_bits_now);
     if (t == 0) finish(result_bits, cb + 1);
 }
 
@@ -741,6 +947,8 @@ constexpr int kTreeParts = 2048;
 
 inline bool is_finite_bits(uint32_t b) { return ((b >> 23) & 0xffu) != 0xffu; }
 
+constexpr size_t kSeqScanLds = (size_t)SEQ_MULTI_LIMIT * 16;  // dynamic LDS of the window-end kernel
+
 // Exact sequential sum (optionally masked) of |x| over n elements.
 int pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold, uint8_t *d_packed,
                  uint64_t *h_survivors, float *h_survivor_sum);
@@ -758,7 +966,8 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     const uint64_t total_blocks = (n + kSeqTile - 1) / kSeqTile;
     void *ws = nullptr;
     // at least 1024 map slots: the window-end kernel reads slot threadIdx.x before it knows the window
-    const uint64_t map_slots = total_blocks > 1024 ? total_blocks : 1024;
+    // and two per block for the windows that span several binades
+    const uint64_t map_slots = total_blocks > 2 * SEQ_MULTI_LIMIT ? total_blocks : 2 * SEQ_MULTI_LIMIT;
     RBN_CHECK(rbn_workspace(ctx, kScratchHeader + map_slots * sizeof(SeqMap) + kMapGrid * 8, &ws));
     ReduceScratch *scr = (ReduceScratch *)ws;
     SeqMap *maps = (SeqMap *)((char *)ws + kScratchHeader);
@@ -775,17 +984,19 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     // sizes the next one by the binades S still has to climb (a window ends where S leaves
     // its binade).
     const unsigned grid = (unsigned)(total_blocks < (uint64_t)kMapGrid ? total_blocks : (uint64_t)kMapGrid);
-    // first batch: S of similar terms climbs one binade per doubling of the position, plus the
-    // first block's window and two spare (a spare pair of launches returns at once: 4 us;
-    // another look by the host costs 10-25 us)
-    int batch = 3;
-    for (uint64_t b = total_blocks; b > 1; b >>= 1) ++batch;
-    batch = batch > 24 ? 24 : batch;
+    // first batch: the binades of the first SEQ_MULTI_LIMIT blocks take three windows (the first
+    // block, and two that carry a pair of maps per block); after them S of similar terms climbs one
+    // binade per doubling of the position; plus one window that ends early and one spare (a spare
+    // pair of launches returns at once: 4 us; another look by the host costs 10-25 us)
+    int batch = 6;
+    RBN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(seq_scan_replay_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSeqScanLds));
+    for (uint64_t b = total_blocks / SEQ_MULTI_LIMIT; b > 1; b >>= 1) ++batch;
     for (;;) {
         for (int i = 0; i < batch; ++i) {
             seq_block_maps_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
                 d_x, n, use_mask, thr, &scr->seq, maps, (uint32_t *)d_packed, count_parts);
-            seq_scan_replay_kernel<<<dim3(1), dim3(1024), 0, ctx->stream>>>(
+            seq_scan_replay_kernel<<<dim3(1), dim3(1024), kSeqScanLds, ctx->stream>>>(
                 maps, d_x, n, total_blocks, use_mask, thr, &scr->seq, h_state, i == batch - 1);
         }
         RBN_HIP(hipGetLastError());

@@ -13,16 +13,25 @@ namespace {
 constexpr int kTile = 4096;
 
 SeqMap thread_map(const float *x, uint64_t base, uint64_t n, uint32_t es, int use_mask, float thr) {
-    SeqMap m = seq_identity();
     const float scale = seq_ulp_scale(es < 26u ? 26u : es);
+    float a[16];
     for (int i = 0; i < 16; ++i) {
         uint64_t idx = base + i;
+        a[i] = 0.0f;  // an element past the end or under the mask: the identity
         if (idx < n) {
-            float a = std::fabs(x[idx]);
-            bool take = use_mask ? (a > thr) : true;
-            if (take) m = seq_append_abs(m, a, es, scale);
+            float v = std::fabs(x[idx]);
+            bool take = use_mask ? (v > thr) : true;
+            if (take) a[i] = v;
         }
     }
+    return seq_map16(a, es, scale);
+}
+
+// The same map term by term (the form seq_map16 falls back to on a tie), for the comparison test.
+SeqMap thread_map_serial(const float *a, uint32_t es) {
+    SeqMap m = seq_identity();
+    const float scale = seq_ulp_scale(es < 26u ? 26u : es);
+    for (int i = 0; i < 16; ++i) m = seq_append_abs(m, a[i], es, scale);
     return m;
 }
 
@@ -107,6 +116,70 @@ ScanResult scan(const std::vector<SeqMap> &maps, uint32_t s_bits) {
 }
 }  // namespace
 
+// The replay of one block (the second half of the window-end kernel): crossings inside the
+// block are resolved one after another.  Returns the state after the block as f32 bits.
+static uint32_t replay_block(const float *x, uint64_t n, uint64_t bbase, int use_mask, float thr,
+                             uint32_t es, uint32_t k_cur) {
+    uint32_t done = 0, result_bits = 0;
+    for (int guard = 0; guard <= 256; ++guard) {
+        SeqMap cm[256], a[256], b2[256];
+        for (int t = 0; t < 256; ++t)
+            cm[t] = (uint32_t)t >= done ? thread_map(x, bbase + (uint64_t)t * 16, n, es, use_mask, thr)
+                                        : seq_identity();
+        for (int t = 0; t < 256; ++t) a[t] = cm[t];
+        SeqMap *src = a, *dst = b2;
+        for (int off = 1; off < 256; off <<= 1) {
+            for (int t = 0; t < 256; ++t) {
+                SeqMap v = src[t];
+                if (t >= off) v = seq_compose(src[t - off], v);
+                dst[t] = v;
+            }
+            std::swap(src, dst);
+        }
+        int tstar = -1;
+        uint32_t kstar = 0;
+        for (int t = 0; t < 256; ++t) {
+            SeqMap before = t == 0 ? seq_identity() : src[t - 1];
+            uint32_t kk = seq_apply(before, k_cur);
+            if ((uint32_t)t >= done && kk < SEQ_K_LIMIT && seq_apply(cm[t], kk) >= SEQ_K_LIMIT) {
+                tstar = t;
+                kstar = kk;
+                break;
+            }
+        }
+        if (tstar < 0) {
+            result_bits = seq_state_join(es, seq_apply(src[255], k_cur));
+            break;
+        }
+        uint32_t jb = seq_state_join(es, kstar);
+        float s;
+        std::memcpy(&s, &jb, 4);
+        for (int i = 0; i < 16; ++i) {
+            uint64_t idx = bbase + (uint64_t)tstar * 16 + i;
+            float av = 0.0f;
+            bool take = false;
+            if (idx < n) {
+                av = std::fabs(x[idx]);
+                take = use_mask ? (av > thr) : true;
+            }
+            volatile float t2 = s + (take ? av : 0.0f);
+            s = t2;
+        }
+        std::memcpy(&result_bits, &s, 4);
+        done = (uint32_t)tstar + 1;
+        if (((result_bits >> 23) & 0xff) == 0xff) {
+            for (uint64_t idx = bbase + (uint64_t)done * 16; idx < bbase + kTile && idx < n; ++idx) {
+                bool take = use_mask ? (std::fabs(x[idx]) > thr) : true;
+                if (take && x[idx] != x[idx]) result_bits |= 0x7fc00000u;
+            }
+            break;
+        }
+        if (done >= 256) break;
+        seq_state_split(result_bits, &es, &k_cur);
+    }
+    return result_bits;
+}
+
 extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr,
                              uint64_t *iterations, uint64_t *elements_read) {
     uint64_t iters = 0, read = 0;
@@ -121,87 +194,53 @@ extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr
     double rate = 0.0;
     while (pos < total_blocks) {
         if (((s_bits >> 23) & 0xff) == 0xff) break;
-        uint32_t es, k;
-        seq_state_split(s_bits, &es, &k);
+        uint32_t es0, k0;
+        seq_state_split(s_bits, &es0, &k0);
         float s_before;
         std::memcpy(&s_before, &s_bits, 4);
-        const uint64_t win = seq_next_window(pos, total_blocks, (double)s_before, rate);
+        uint32_t multi = 0;
+        const uint64_t win = seq_plan_window(pos, total_blocks, (double)s_before, rate, &multi);
+        const uint32_t rate_lo = seq_multi_rate_lo(rate);
+        const uint32_t nm = multi ? 2u : 1u;
         const uint64_t first = pos * kTile;
-        std::vector<SeqMap> maps(win);
-        for (uint64_t b = 0; b < win; ++b) maps[b] = block_map(x, first + b * kTile, n, es, use_mask, thr);
-        read += win * kTile;
-        ScanResult sr = scan(maps, s_bits);
-        uint64_t next_rel;
-        if (sr.cross_block == 0xffffffffu) {
-            s_bits = seq_state_join(es, sr.k);
-            next_rel = win;
-        } else {
-            // the replay kernel: crossings inside the block are resolved one after another
-            const uint64_t bbase = first + (uint64_t)sr.cross_block * kTile;
-            uint32_t k_cur = sr.k, done = 0, result_bits = 0;
-            for (int guard = 0; guard <= 256; ++guard) {
-                SeqMap cm[256], a[256], b2[256];
-                for (int t = 0; t < 256; ++t)
-                    cm[t] = (uint32_t)t >= done ? thread_map(x, bbase + (uint64_t)t * 16, n, es, use_mask, thr)
-                                                : seq_identity();
-                for (int t = 0; t < 256; ++t) a[t] = cm[t];
-                SeqMap *src = a, *dst = b2;
-                for (int off = 1; off < 256; off <<= 1) {
-                    for (int t = 0; t < 256; ++t) {
-                        SeqMap v = src[t];
-                        if (t >= off) v = seq_compose(src[t - off], v);
-                        dst[t] = v;
-                    }
-                    std::swap(src, dst);
-                }
-                int tstar = -1;
-                uint32_t kstar = 0;
-                for (int t = 0; t < 256; ++t) {
-                    SeqMap before = t == 0 ? seq_identity() : src[t - 1];
-                    uint32_t kk = seq_apply(before, k_cur);
-                    if ((uint32_t)t >= done && kk < SEQ_K_LIMIT && seq_apply(cm[t], kk) >= SEQ_K_LIMIT) {
-                        tstar = t;
-                        kstar = kk;
-                        break;
-                    }
-                }
-                if (tstar < 0) {
-                    result_bits = seq_state_join(es, seq_apply(src[255], k_cur));
-                    break;
-                }
-                uint32_t jb = seq_state_join(es, kstar);
-                float s;
-                std::memcpy(&s, &jb, 4);
-                for (int i = 0; i < 16; ++i) {
-                    uint64_t idx = bbase + (uint64_t)tstar * 16 + i;
-                    float av = 0.0f;
-                    bool take = false;
-                    if (idx < n) {
-                        av = std::fabs(x[idx]);
-                        take = use_mask ? (av > thr) : true;
-                    }
-                    volatile float t2 = s + (take ? av : 0.0f);
-                    s = t2;
-                }
-                std::memcpy(&result_bits, &s, 4);
-                done = (uint32_t)tstar + 1;
-                if (((result_bits >> 23) & 0xff) == 0xff) {
-                    for (uint64_t idx = bbase + (uint64_t)done * 16; idx < bbase + kTile && idx < n; ++idx) {
-                        bool take = use_mask ? (std::fabs(x[idx]) > thr) : true;
-                        if (take && x[idx] != x[idx]) result_bits |= 0x7fc00000u;
-                    }
-                    break;
-                }
-                if (done >= 256) break;
-                seq_state_split(result_bits, &es, &k_cur);
-            }
-            s_bits = result_bits;
-            next_rel = sr.cross_block + 1;
+        // the maps kernel: one map per block for the state's exponent, or two for the pair that the
+        // prediction gives the block
+        std::vector<uint32_t> elo(win);
+        std::vector<SeqMap> maps(win * nm);
+        for (uint64_t b = 0; b < win; ++b) {
+            elo[b] = multi ? seq_multi_es_lo(s_bits, rate_lo, (uint32_t)b) : es0;
+            for (uint32_t j = 0; j < nm; ++j)
+                maps[b * nm + j] = block_map(x, first + b * kTile, n, elo[b] + j, use_mask, thr);
         }
+        read += win * kTile;
+        // the window-end kernel: scan to the crossing, replay that block, go on in the new binade
+        // while the blocks' maps hold it
+        uint64_t b_cur = 0;
+        uint32_t cur_bits = s_bits;
+        for (int guard = 0; guard < 64; ++guard) {
+            uint32_t es, k;
+            seq_state_split(cur_bits, &es, &k);
+            uint64_t range_end = b_cur;
+            while (range_end < win && es >= elo[range_end] && es - elo[range_end] < nm) ++range_end;
+            if (range_end == b_cur) break;
+            std::vector<SeqMap> sel(range_end - b_cur);
+            for (uint64_t b = b_cur; b < range_end; ++b) sel[b - b_cur] = maps[b * nm + (es - elo[b])];
+            ScanResult sr = scan(sel, cur_bits);
+            if (sr.cross_block == 0xffffffffu) {
+                cur_bits = seq_state_join(es, sr.k);
+                b_cur = range_end;
+                break;
+            }
+            cur_bits = replay_block(x, n, first + (b_cur + sr.cross_block) * kTile, use_mask, thr, es, sr.k);
+            b_cur += (uint64_t)sr.cross_block + 1;
+            if (((cur_bits >> 23) & 0xff) == 0xff || b_cur >= win) break;
+        }
+        if (b_cur == 0) return NAN;  // no progress: cannot happen (block 0 holds the state's exponent)
+        s_bits = cur_bits;
         float s_after;
         std::memcpy(&s_after, &s_bits, 4);
-        rate = ((double)s_after - (double)s_before) / (double)next_rel;
-        pos += next_rel;
+        rate = ((double)s_after - (double)s_before) / (double)b_cur;
+        pos += b_cur;
         ++iters;
     }
     float s;
@@ -231,6 +270,54 @@ extern "C" float seqsum_literal(const float *x, uint64_t n, int use_mask, float 
         if (take) s = s + a;
     }
     return s;
+}
+
+// seq_map16 against sixteen seq_append_abs on `count` pseudo-random groups of sixteen terms around
+// the state's ulp (short mantissas, so that ties happen; zeros, huge terms, Inf and NaN among them).
+// Returns the number of disagreements (both at or above the limit counts as agreement).
+extern "C" uint64_t seqsum_compare_map16(uint64_t count, uint64_t seed, uint64_t *groups_with_a_tie) {
+    uint64_t bad = 0, ties = 0, x = seed * 0x9E3779B97F4A7C15ull + 1;
+    auto next = [&]() {
+        x ^= x << 13;
+        x ^= x >> 7;
+        x ^= x << 17;
+        return x;
+    };
+    for (uint64_t g = 0; g < count; ++g) {
+        const uint32_t es = 20u + (uint32_t)(next() % 235u);  // 20 .. 254: both term splits
+        float a[16];
+        for (int i = 0; i < 16; ++i) {
+            uint32_t ex = es - 27u + (uint32_t)(next() % 30u);  // ulp/8 .. far above
+            if (ex > 255u) ex = 0u;
+            uint32_t frac = (uint32_t)(next() & 0x7fffffu);
+            switch (next() % 8u) {
+                case 0: frac = 0; break;
+                case 1: frac &= 0x700000u; break;
+                case 2: frac = 0x400000u; break;
+                case 3: ex = 0; frac = 0; break;            // +0.0
+                case 4: if (next() % 64u == 0) ex = 255u; break;  // Inf / NaN now and then
+                default: break;
+            }
+            const uint32_t bits = (ex << 23) | frac;
+            std::memcpy(&a[i], &bits, 4);
+        }
+        const float scale = seq_ulp_scale(es < 26u ? 26u : es);
+        bool tie = false;
+        for (int i = 0; i < 16 && es >= 26u; ++i) {
+            const float v = a[i] * scale;
+            if (v < 33554432.0f && v - std::floor(v) == 0.5f) tie = true;
+        }
+        ties += tie ? 1 : 0;
+        const SeqMap want = thread_map_serial(a, es), got = seq_map16(a, es, scale);
+        const bool w_over = want.d0 >= SEQ_K_LIMIT / 2 || want.d1 >= SEQ_K_LIMIT / 2;
+        if (w_over) {
+            if (got.d0 < SEQ_K_LIMIT / 2 || got.d1 < SEQ_K_LIMIT / 2) ++bad;
+        } else if (got.d0 != want.d0 || got.d1 != want.d1) {
+            ++bad;
+        }
+    }
+    if (groups_with_a_tie) *groups_with_a_tie = ties;
+    return bad;
 }
 
 // Compares the floating-point term split (seq_append_abs, es >= 26) with the integer one

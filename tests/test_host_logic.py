@@ -119,6 +119,8 @@ def seqsum(tmp_path_factory):
     L.seqsum_literal.argtypes = [C.c_void_p, C.c_uint64, C.c_int, C.c_float]
     L.seqsum_compare_term_splits.restype = C.c_uint64
     L.seqsum_compare_term_splits.argtypes = [C.c_uint64, C.c_uint64]
+    L.seqsum_compare_map16.restype = C.c_uint64
+    L.seqsum_compare_map16.argtypes = [C.c_uint64, C.c_uint64, C.POINTER(C.c_uint64)]
     return L
 
 
@@ -163,6 +165,13 @@ def test_float_and_integer_term_splits_agree(seqsum):
     # seq_append_abs (float split, used for es >= 26) against seq_append (integer split)
     assert seqsum.seqsum_compare_term_splits(3_000_000, 1) == 0
     assert seqsum.seqsum_compare_term_splits(1_000_000, 2) == 0
+
+
+def test_map_of_sixteen_terms_equals_term_by_term(seqsum):
+    # seq_map16 (one sum of sixteen roundings unless a term is an exact tie) against sixteen seq_append_abs
+    ties = C.c_uint64()
+    assert seqsum.seqsum_compare_map16(400_000, 5, C.byref(ties)) == 0
+    assert 1000 < ties.value < 399_000      # both branches were taken
 
 
 def test_sequential_sum_traffic_is_bounded(seqsum):

@@ -151,16 +151,21 @@ SEQ_HD SeqMap seq_append_abs(SeqMap m, float a, uint32_t es, float scale) {
 // when none of the sixteen is such a tie (the rule: a tie needs a term whose low bits are exactly
 // 1000...0 at the state's ulp), the map is one sum of sixteen independent roundings, d0 = d1, and
 // the sixteen terms do not wait for each other as they do in seq_append_abs; with a tie among them
-// the terms are appended one by one.  v is clamped to 2^25 = SEQ_SAT first (NaN included: the
-// minimum of a NaN and a number is the number), so a sum of sixteen stays below 2^32 and a term far
-// above the binade saturates the map exactly as it does in seq_append_abs.
+// the terms are appended one by one.  v is clamped to 2^25 = SEQ_SAT first (NaN included), so a
+// sum of sixteen stays below 2^32 and a term far above the binade saturates the map exactly as it
+// does in seq_append_abs.
 SEQ_HD SeqMap seq_map16(const float *a, uint32_t es, float scale) {
     SeqMap m = seq_identity();
     bool tie = es < 26u;  // below that the term is split in integer arithmetic
     if (!tie) {
         uint32_t sum = 0u;
         for (int i = 0; i < 16; ++i) {
-            const float v = __builtin_fminf(a[i] * scale, 33554432.0f);
+            // the clamp on the bit patterns: for v >= +0 they order as the values do, NaNs above all
+            float v = a[i] * scale;
+            uint32_t vb;
+            __builtin_memcpy(&vb, &v, 4);
+            vb = seq_min_u32(vb, 0x4c000000u);  // 2^25
+            __builtin_memcpy(&v, &vb, 4);
             const float r = __builtin_rintf(v);  // to nearest, ties to even (the default rounding mode)
             tie = tie || __builtin_fabsf(v - r) == 0.5f;
             sum += (uint32_t)r;
@@ -202,7 +207,7 @@ SEQ_HD uint64_t seq_next_window(uint64_t pos, uint64_t total_blocks, double s_no
         int e = 0;
         (void)frexp(s_now, &e);  // s_now = m * 2^e, m in [0.5, 1): the binade ends at 2^e
         const double need = (ldexp(1.0, e) - s_now) / rate;
-        win = need < 1e15 ? (uint64_t)(need * 1.06) + 4u : total_blocks;
+        win = need < 1e15 ? (uint64_t)(need * 1.10) + 4u : total_blocks;
     }
     if (win < 64u) win = 64u;
     if (win > total_blocks - pos) win = total_blocks - pos;

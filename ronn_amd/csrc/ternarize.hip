@@ -246,6 +246,7 @@ struct SeqState {
     uint64_t fresh_from;  // blocks from here on have not been seen by any window yet
     uint32_t rate_lo;   // multi: the cautious growth of S per block (f32 bits) behind the blocks' exponents
     uint32_t pad;
+    uint64_t survivors;  // packing sums only: elements above the threshold, set by the window that ends the sum
 };
 
 // A SeqMap from another lane by a DPP move: lanes without a source (and rows outside the
@@ -327,7 +328,20 @@ __device__ __forceinline__ void seq_block_maps_body(
     if (MULTI) mb = seq_map16(am, es + 1u, scale_b);
     // ordered reduction of the wave by DPP moves (each lane absorbs what lies to its left):
     // lane 63 ends up with the map of all 1024 elements
+    // (maps that do not depend on the parity of k - all of them unless a term is an exact tie -
+    // compose by adding their increments, in any order: one DPP add per step)
     auto wave_fold = [](SeqMap v) {
+        if (__ballot(v.d0 != v.d1) == 0ull) {
+            int sum = (int)v.d0;  // <= 2^25 per lane: a wave's total stays below 2^31
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x111, 0xf, 0xf, true);  // row_shr:1
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x112, 0xf, 0xf, true);  // row_shr:2
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x114, 0xf, 0xf, true);  // row_shr:4
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x118, 0xf, 0xf, true);  // row_shr:8
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x142, 0xa, 0xf, true);  // row_bcast15
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x143, 0xc, 0xf, true);  // row_bcast31
+            v.d0 = v.d1 = seq_min_u32((uint32_t)sum, SEQ_SAT);
+            return v;
+        }
         v = seq_compose(seq_dpp<0x111, 0xf>(v), v);  // row_shr:1
         v = seq_compose(seq_dpp<0x112, 0xf>(v), v);  // row_shr:2
         v = seq_compose(seq_dpp<0x114, 0xf>(v), v);  // row_shr:4
@@ -378,36 +392,26 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
     __shared__ SeqMap s_wave[2 * (kBlock / 64)];
     __shared__ unsigned s_cnt[kBlock / 64];
     if (state->done) return;
+    // (plain loads also in long windows: a thread's four loads share their cache lines, and
+    // non-temporal ones fetched each line four times - 98 -> 130 us for the last window of 8192 x 28672)
     if (state->multi)
         seq_block_maps_body<true>(x, n, use_mask, thr, state, maps, packed, count_parts, s_wave, s_cnt);
     else
         seq_block_maps_body<false>(x, n, use_mask, thr, state, maps, packed, count_parts, s_wave, s_cnt);
 }
 
-__global__ __launch_bounds__(kBlock) void fill_u64_kernel(unsigned long long *p, int n) {
-    for (int i = threadIdx.x; i < n; i += kBlock) p[i] = 0;
-}
-__global__ __launch_bounds__(kBlock) void sum_u64_kernel(const unsigned long long *__restrict__ p, int n,
-                                                        unsigned long long *__restrict__ out) {
-    __shared__ unsigned long long s[kBlock];
-    unsigned long long acc = 0;
-    for (int i0 = 0; i0 < n; i0 += 8 * kBlock) {  // eight loads in flight per thread
-        unsigned long long v[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int i = i0 + j * kBlock + (int)threadIdx.x;
-            v[j] = p[i < n ? i : n - 1];
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc += (i0 + j * kBlock + (int)threadIdx.x) < n ? v[j] : 0ull;
+// The state before the first window (one launch instead of a fill and a copy from the host): S = +0,
+// nothing folded, the first window `win0` blocks long; the per-workgroup survivor counters cleared.
+__global__ __launch_bounds__(kBlock) void seq_init_kernel(SeqState *__restrict__ state, uint32_t win0,
+                                                         unsigned long long *__restrict__ count_parts, int n_parts) {
+    if (count_parts)
+        for (int i = threadIdx.x; i < n_parts; i += kBlock) count_parts[i] = 0;
+    if (threadIdx.x == 0) {
+        SeqState z;
+        z.s_bits = 0, z.win = win0, z.pos = 0, z.done = 0, z.error = 0, z.saw_nan = 0, z.multi = 0;
+        z.fresh_from = 0, z.rate_lo = 0, z.pad = 0, z.survivors = 0;
+        *state = z;
     }
-    s[threadIdx.x] = acc;
-    __syncthreads();
-    for (int off = kBlock / 2; off > 0; off >>= 1) {
-        if ((int)threadIdx.x < off) s[threadIdx.x] += s[threadIdx.x + off];
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) *out = s[0];
 }
 
 // Ordered scans of SeqMaps without a barrier per step: inside a wave by shuffles (lane l
@@ -464,12 +468,25 @@ __device__ __forceinline__ SeqMap seq_block_before(SeqMap m, SeqMap *s_w, SeqMap
 // touches them again.
 __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x, uint64_t n, uint64_t block_base,
                                                      int use_mask, float thr, uint32_t es, uint32_t k_cur,
-                                                     SeqMap *s_w, unsigned *s_first, uint32_t *s_bits_now) {
+                                                     SeqMap *s_w, unsigned *s_first, uint32_t *s_bits_now,
+                                                     float *s_head /* 128 floats */) {
     const uint32_t t = threadIdx.x;
     constexpr int NW = kBlock / 64;
     const bool worker = __builtin_amdgcn_readfirstlane((int)(t >> 6)) < NW;  // wave-uniform
+    // A sum that starts at zero doubles every few elements: crossed binade by binade, the first
+    // 128 elements cost seven turns of the loop below.  They are added one after the other instead
+    // (that IS the fold, so it is exact whatever the state).
+    const bool head = es == 1u && k_cur == 0u;
     if (!worker) {
-        // the barriers of the loop below, in the same order, and its exits
+        // the barriers of the worker waves, in the same order, and their exits
+        if (head) {
+            __syncthreads();  // (h1) head elements in LDS
+            __syncthreads();  // (h2) head folded
+            if (((*s_bits_now >> 23) & 0xffu) == 0xffu) {
+                __syncthreads();  // (h3) NaN behind an Inf
+                return 0u;
+            }
+        }
         for (int guard = 0; guard <= kBlock; ++guard) {
             __syncthreads();  // (1) wave totals written
             __syncthreads();  // (2) crossing chunk known
@@ -508,6 +525,40 @@ __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x
     const int lane = t & 63, wave = t >> 6;
     uint32_t done = 0;  // chunks [0, done) are already folded into (es, k_cur)
     uint32_t result_bits = 0;
+    if (head) {
+        constexpr uint32_t kHeadChunks = 8;
+        if (t < kHeadChunks) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s_head[t * 16 + i] = a[i];
+        }
+        __syncthreads();  // (h1)
+        if (t == 0) {
+            float sum = __uint_as_float(seq_state_join(es, k_cur));
+            for (uint32_t i = 0; i < kHeadChunks * 16; i += 4) {
+                const float4 v = *reinterpret_cast<const float4 *>(s_head + i);
+                sum = sum + v.x;
+                sum = sum + v.y;
+                sum = sum + v.z;
+                sum = sum + v.w;
+            }
+            *s_bits_now = __float_as_uint(sum);
+        }
+        __syncthreads();  // (h2)
+        result_bits = *s_bits_now;
+        done = kHeadChunks;
+        if (((result_bits >> 23) & 0xffu) == 0xffu) {
+            // as below: +Inf turns into NaN if a NaN follows inside this block
+            bool nan_after = false;
+            if (t >= done) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) nan_after |= (a[i] != a[i]);
+            }
+            if (nan_after) atomicOr(s_bits_now, 0x7fc00000u);
+            __syncthreads();  // (h3)
+            return *s_bits_now;  // (already in LDS for the other waves)
+        }
+        seq_state_split(result_bits, &es, &k_cur);
+    }
     for (int guard = 0; guard <= kBlock; ++guard) {
         SeqMap m = seq_identity();
         if (t >= done) m = seq_map16(a, es, seq_ulp_scale(es < 26u ? 26u : es));
@@ -592,7 +643,9 @@ __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x
 __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     const SeqMap *__restrict__ maps, const float *__restrict__ x, uint64_t n, uint64_t total_blocks,
     int use_mask, float thr, SeqState *__restrict__ state, SeqState *__restrict__ host_copy,
-    int mirror /* the last launch of a batch: the host reads the state after it */) {
+    int mirror /* the last launch of a batch: the host reads the state after it */,
+    const unsigned long long *__restrict__ count_parts /* packing sums: the maps kernels' survivor counters */,
+    int n_parts) {
     extern __shared__ uint4 s_maps[];  // SEQ_MULTI_LIMIT units: the maps of a window with two per block
     __shared__ SeqMap s_w[16];
     __shared__ unsigned s_first;
@@ -600,6 +653,8 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     __shared__ uint32_t s_bits_now;
     __shared__ unsigned long long s_min64;
     __shared__ uint32_t s_edge[64];
+    __shared__ unsigned long long s_cnt64[16];
+    __shared__ __attribute__((aligned(16))) float s_head[128];
     const uint32_t t = threadIdx.x;
     // Windows of up to 1024 blocks (most of them) have one map per thread: it is requested
     // here, before the state is known, so that the two round trips overlap (the buffer holds
@@ -620,6 +675,23 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     seq_state_split(bits0, &es, &k0);
     // ends the window: the state after `advanced` blocks, the next window's size from the
     // growth of S over this one, mirrored to the host
+    // The window that folds the last block also adds up the survivor counters of the packing pass
+    // (all maps kernels have run by then): called by every thread with the same `advanced`, before
+    // finish(); the total is valid in thread 0.
+    unsigned long long survivors_total = 0;
+    auto count_survivors = [&](uint32_t advanced) {
+        if (count_parts == nullptr || pos0 + advanced < total_blocks) return;
+        unsigned long long acc = 0;
+        for (int i = (int)t; i < n_parts; i += 1024) acc += count_parts[i];
+        for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off);
+        if ((t & 63u) == 0) s_cnt64[t >> 6] = acc;
+        __syncthreads();
+        if (t == 0) {
+            unsigned long long sum = 0;
+            for (int w = 0; w < 16; ++w) sum += s_cnt64[w];
+            survivors_total = sum;
+        }
+    };
     auto finish = [&](uint32_t bits, uint32_t advanced) {
         const uint64_t pos = pos0 + advanced;
         const bool finite = ((bits >> 23) & 0xffu) != 0xffu;
@@ -636,6 +708,7 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         next.rate_lo = seq_multi_rate_lo(rate);
         next.saw_nan = 0;
         next.pad = 0;
+        next.survivors = survivors_total;
         const uint64_t seen = pos0 + nblocks, before = state->fresh_from;
         next.fresh_from = seen > before ? seen : before;
         *state = next;
@@ -736,12 +809,13 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
             }
             const uint32_t cb = (uint32_t)(first_cross >> 32), k_cb = (uint32_t)first_cross;
             (void)seq_replay_block(x, n, first + (uint64_t)cb * kSeqTile, use_mask, thr, es, k_cb, s_w, &s_first,
-                                   &s_bits_now);
+                                   &s_bits_now, s_head);
             __syncthreads();  // the result is in LDS; s_w and s_min64 are rewritten in the next turn
             cur_bits = s_bits_now;
             b_cur = cb + 1u;
             if (((cur_bits >> 23) & 0xffu) == 0xffu || b_cur >= nblocks) break;
         }
+        count_survivors(b_cur);
         if (t == 0) finish(cur_bits, b_cur);
         return;
     }
@@ -844,13 +918,15 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     const uint32_t cb = s_cross_block;
     uint32_t k_cur = s_cross_k;
     if (cb == 0xffffffffu) {
+        count_survivors(nblocks);
         if (t == 0) finish(seq_state_join(es, k_cur), nblocks);
         return;
     }
 
     // ---- (2) replay of block cb
     const uint32_t result_bits = seq_replay_block(x, n, first + (uint64_t)cb * kSeqTile, use_mask, thr, es, k_cur,
-                                                  s_w, &s_first, &s_bits_now);
+                                                  s_w, &s_first, &s_bits_now, s_head);
+    count_survivors(cb + 1);
     if (t == 0) finish(result_bits, cb + 1);
 }
 
@@ -973,12 +1049,10 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     SeqMap *maps = (SeqMap *)((char *)ws + kScratchHeader);
     unsigned long long *count_parts =
         d_packed ? (unsigned long long *)((char *)ws + kScratchHeader + map_slots * sizeof(SeqMap)) : nullptr;
-    if (d_packed) fill_u64_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(count_parts, kMapGrid);
     SeqState *h_state = (SeqState *)ctx->mailbox;
     memset(h_state, 0, sizeof(SeqState));
-    h_state->win = (uint32_t)seq_next_window(0, total_blocks, 0.0, 0.0);
-    RBN_HIP(hipMemcpyAsync(&scr->seq, h_state, sizeof(SeqState), hipMemcpyHostToDevice,
-                           ctx->stream));
+    seq_init_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(
+        &scr->seq, (uint32_t)seq_next_window(0, total_blocks, 0.0, 0.0), count_parts, kMapGrid);
     // Windows are queued in batches: the kernels take each window from the device state and
     // return at once when the sum is complete, so the host only looks in between batches and
     // sizes the next one by the binades S still has to climb (a window ends where S leaves
@@ -986,9 +1060,9 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     const unsigned grid = (unsigned)(total_blocks < (uint64_t)kMapGrid ? total_blocks : (uint64_t)kMapGrid);
     // first batch: the binades of the first SEQ_MULTI_LIMIT blocks take three windows (the first
     // block, and two that carry a pair of maps per block); after them S of similar terms climbs one
-    // binade per doubling of the position; plus one window that ends early and one spare (a spare
+    // binade per doubling of the position; plus one more (a window that ends early, or a spare
     // pair of launches returns at once: 4 us; another look by the host costs 10-25 us)
-    int batch = 6;
+    int batch = 5;
     RBN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(seq_scan_replay_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSeqScanLds));
     for (uint64_t b = total_blocks / SEQ_MULTI_LIMIT; b > 1; b >>= 1) ++batch;
@@ -997,7 +1071,8 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
             seq_block_maps_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
                 d_x, n, use_mask, thr, &scr->seq, maps, (uint32_t *)d_packed, count_parts);
             seq_scan_replay_kernel<<<dim3(1), dim3(1024), kSeqScanLds, ctx->stream>>>(
-                maps, d_x, n, total_blocks, use_mask, thr, &scr->seq, h_state, i == batch - 1);
+                maps, d_x, n, total_blocks, use_mask, thr, &scr->seq, h_state, i == batch - 1, count_parts,
+                (int)grid);
         }
         RBN_HIP(hipGetLastError());
         RBN_HIP(hipStreamSynchronize(ctx->stream));
@@ -1033,12 +1108,8 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
             // the sum left the finite range before the end: the windows stopped there, so
             // pack (and count) with the plain kernel
             RBN_CHECK(pack_ternary(ctx, d_x, n, thr, d_packed, h_survivors, nullptr));
-        } else {
-            sum_u64_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(count_parts, (int)grid, &scr->survivors);
-            RBN_HIP(hipGetLastError());
-            RBN_HIP(hipMemcpyAsync(ctx->mailbox, &scr->survivors, 8, hipMemcpyDeviceToHost, ctx->stream));
-            RBN_HIP(hipStreamSynchronize(ctx->stream));
-            if (h_survivors) memcpy(h_survivors, ctx->mailbox, 8);
+        } else if (h_survivors) {
+            *h_survivors = h_state->survivors;  // added up by the window that folded the last block
         }
     }
     return RBN_OK;

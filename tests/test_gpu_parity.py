@@ -100,6 +100,29 @@ def test_strict_abs_sum_matches_sequential_fold(ctx, dist, n):
         assert bits(got_m) == bits(want_m)
 
 
+def _steps(n, seed):
+    """Growth that changes by orders of magnitude along the tensor: the windows that predict the
+    exponent of S per block lose it in both directions and must end early, not go wrong."""
+    x = synth_normal(seed, 1.0, (n,))
+    scale = np.ones(n, dtype=np.float32)
+    cuts = [0, n // 16, n // 7, n // 3, n // 2, (3 * n) // 4, n]
+    for i, f in enumerate((1e-6, 1.0, 1e-3, 300.0, 0.0, 2e-2)):
+        scale[cuts[i]:cuts[i + 1]] = f
+    return (x * scale).astype(np.float32)
+
+
+@pytest.mark.parametrize("n", [300_001, 3_000_000])
+def test_strict_abs_sum_when_the_growth_prediction_fails(ctx, n):
+    x = _steps(n, 21)
+    want = np.cumsum(np.abs(x), dtype=np.float32)[-1]
+    got, cnt = ctx.abs_sum(ctx.to_device(x), n, STRICT)
+    assert bits(got) == bits(want) and cnt == n
+    thr = np.float32(1e-3)
+    surv = np.abs(x)[np.abs(x) > thr]
+    got_m, cnt_m = ctx.abs_sum(ctx.to_device(x), n, STRICT, mask_threshold=thr)
+    assert cnt_m == surv.size and bits(got_m) == bits(np.cumsum(surv, dtype=np.float32)[-1])
+
+
 def test_strict_abs_sum_nonfinite(ctx):
     x = synth_normal(9, 1.0, (100000,))
     for edit, want in (({5000: np.inf}, np.inf), ({5000: np.inf, 90000: np.nan}, np.nan),

@@ -143,6 +143,12 @@ def _cases():
     yield "inf_then_nan_same_block", x
     x = rng.normal(0, 1, 100000); x[70000] = np.nan
     yield "nan", x
+    # growth that changes by orders of magnitude: the exponent prediction of the multi-binade windows fails
+    x = rng.normal(0, 1, 700000)
+    for lo, hi, f in ((0, 40000, 1e-6), (40000, 100000, 1.0), (100000, 230000, 1e-3), (230000, 350000, 300.0),
+                      (350000, 520000, 0.0), (520000, 700000, 2e-2)):
+        x[lo:hi] *= f
+    yield "steps", x
     yield "lognormal", rng.lognormal(0, 6, 500000)
     yield "cauchy", np.abs(rng.standard_cauchy(300000))
     yield "ties_even", np.concatenate([[2.0 ** 20], np.full(300000, 2.0 ** -4)])

@@ -267,9 +267,11 @@ __device__ __forceinline__ SeqMap seq_dpp(SeqMap m) {
 // every block that no earlier window has touched - a thread's 16 elements are one 32-bit word
 // of the reference's layout - and adds their survivors to this workgroup's counter: the
 // scale's sum and the packing then share one pass over the tensor.
-template <bool MULTI>
+// MASK and PACK are compile-time copies of use_mask and packed != nullptr: the body is the same,
+// without the run-time selects per element.
+template <bool MULTI, bool MASK, bool PACK>
 __device__ __forceinline__ void seq_block_maps_body(
-    const float *__restrict__ x, uint64_t n, int use_mask, float thr,
+    const float *__restrict__ x, uint64_t n, float thr,
     const SeqState *__restrict__ state, SeqMap *__restrict__ maps, uint32_t *__restrict__ packed,
     unsigned long long *__restrict__ count_parts, SeqMap *s_wave, unsigned *s_cnt) {
     const uint32_t win = state->win;
@@ -284,7 +286,7 @@ __device__ __forceinline__ void seq_block_maps_body(
     const float scale = seq_ulp_scale(es < 26u ? 26u : es);
     const float scale_b = seq_ulp_scale(es + 1u < 26u ? 26u : es + 1u);
     uint64_t base = first + (uint64_t)blk * kSeqTile + (uint64_t)threadIdx.x * 16;
-    const bool fresh = packed != nullptr && pos + blk >= fresh_from;
+    const bool fresh = PACK && pos + blk >= fresh_from;
     uint32_t word = 0;
     float am[16];  // |x| of the elements that count, +0.0 (the identity as a term) for the others
     if (base + 16 <= n) {
@@ -297,7 +299,7 @@ __device__ __forceinline__ void seq_block_maps_body(
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 float a = fabsf(e[i]);
-                bool take = use_mask ? (a > thr) : true;
+                bool take = MASK ? (a > thr) : true;
                 am[4 * j + i] = take ? a : 0.0f;
                 if (fresh) {
                     word |= ternary_code(e[i], thr) << (2 * (4 * j + i));
@@ -314,7 +316,7 @@ __device__ __forceinline__ void seq_block_maps_body(
             if (idx < n) {
                 float e = x[idx];
                 float a = fabsf(e);
-                bool take = use_mask ? (a > thr) : true;
+                bool take = MASK ? (a > thr) : true;
                 am[i] = take ? a : 0.0f;
                 if (fresh) {
                     word |= ternary_code(e, thr) << (2 * i);
@@ -371,7 +373,7 @@ __device__ __forceinline__ void seq_block_maps_body(
     }
     __syncthreads();  // s_wave is rewritten in the next turn
   }
-    if (packed) {
+    if (PACK) {
         // one plain read-modify-write per workgroup and launch: slot blockIdx.x belongs to
         // this workgroup alone, and launches are ordered by the stream
         for (int off = 32; off > 0; off >>= 1) fresh_count += __shfl_down(fresh_count, off);
@@ -394,10 +396,19 @@ __global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
     if (state->done) return;
     // (plain loads also in long windows: a thread's four loads share their cache lines, and
     // non-temporal ones fetched each line four times - 98 -> 130 us for the last window of 8192 x 28672)
+    auto run = [&](auto multi) {
+        constexpr bool M = decltype(multi)::value;
+        if (packed != nullptr)  // packing goes with a masked sum (thr is the ternary threshold)
+            seq_block_maps_body<M, true, true>(x, n, thr, state, maps, packed, count_parts, s_wave, s_cnt);
+        else if (use_mask)
+            seq_block_maps_body<M, true, false>(x, n, thr, state, maps, packed, count_parts, s_wave, s_cnt);
+        else
+            seq_block_maps_body<M, false, false>(x, n, thr, state, maps, packed, count_parts, s_wave, s_cnt);
+    };
     if (state->multi)
-        seq_block_maps_body<true>(x, n, use_mask, thr, state, maps, packed, count_parts, s_wave, s_cnt);
+        run(std::true_type{});
     else
-        seq_block_maps_body<false>(x, n, use_mask, thr, state, maps, packed, count_parts, s_wave, s_cnt);
+        run(std::false_type{});
 }
 
 // The state before the first window (one launch instead of a fill and a copy from the host): S = +0,

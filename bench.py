@@ -758,6 +758,7 @@ def main():
                                  "roofline": {"bound": "mfma", "achieved": ops / (ms * 1e-3) / 1e12,
                                               "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                                               "frac": ops / (ms * 1e-3) / 1e12 / INT8_PEAK_TOPS,
+                                              "traffic": gfacts.get("traffic_bytes_per_launch"),
                                               "kernel": gfacts.get("kernel", "gemm_t2_i8_mfma_kernel")}}
         del pw, pwt
         extra["act_quant_i8"] = time_act_quant(ctx)

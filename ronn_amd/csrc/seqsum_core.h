@@ -154,26 +154,37 @@ SEQ_HD SeqMap seq_append_abs(SeqMap m, float a, uint32_t es, float scale) {
 // the terms are appended one by one.  v is clamped to 2^25 = SEQ_SAT first (NaN included), so a
 // sum of sixteen stays below 2^32 and a term far above the binade saturates the map exactly as it
 // does in seq_append_abs.
+// Maps without a tie are plain increments (d0 = d1), and composing increments is adding them, in any
+// order and any grouping: as long as no term of a whole block is a tie, the block's map is the
+// (saturated) sum of all its roundings however its elements are dealt to the threads.
+//
+// The sum of the sixteen roundings, and in *tie whether it may NOT be used: a term is an exact tie,
+// or es < 26 (there the term is split in integer arithmetic, by seq_append).
+SEQ_HD uint32_t seq_sum16(const float *a, uint32_t es, float scale, bool *tie) {
+    bool t = es < 26u;
+    uint32_t sum = 0u;
+    for (int i = 0; i < 16; ++i) {
+        // the clamp on the bit patterns: for v >= +0 they order as the values do, NaNs above all
+        float v = a[i] * scale;
+        uint32_t vb;
+        __builtin_memcpy(&vb, &v, 4);
+        vb = seq_min_u32(vb, 0x4c000000u);  // 2^25
+        __builtin_memcpy(&v, &vb, 4);
+        const float r = __builtin_rintf(v);  // to nearest, ties to even (the default rounding mode)
+        t = t || __builtin_fabsf(v - r) == 0.5f;
+        sum += (uint32_t)r;
+    }
+    *tie = t;
+    return sum;
+}
+
 SEQ_HD SeqMap seq_map16(const float *a, uint32_t es, float scale) {
     SeqMap m = seq_identity();
-    bool tie = es < 26u;  // below that the term is split in integer arithmetic
+    bool tie;
+    const uint32_t sum = seq_sum16(a, es, scale, &tie);
     if (!tie) {
-        uint32_t sum = 0u;
-        for (int i = 0; i < 16; ++i) {
-            // the clamp on the bit patterns: for v >= +0 they order as the values do, NaNs above all
-            float v = a[i] * scale;
-            uint32_t vb;
-            __builtin_memcpy(&vb, &v, 4);
-            vb = seq_min_u32(vb, 0x4c000000u);  // 2^25
-            __builtin_memcpy(&v, &vb, 4);
-            const float r = __builtin_rintf(v);  // to nearest, ties to even (the default rounding mode)
-            tie = tie || __builtin_fabsf(v - r) == 0.5f;
-            sum += (uint32_t)r;
-        }
         m.d0 = m.d1 = seq_min_u32(sum, SEQ_SAT);
-    }
-    if (tie) {
-        m = seq_identity();
+    } else {
         for (int i = 0; i < 16; ++i) m = seq_append_abs(m, a[i], es, scale);
     }
     return m;

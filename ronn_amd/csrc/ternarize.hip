@@ -286,7 +286,97 @@ __device__ __forceinline__ void seq_block_maps_body(
     const float scale = seq_ulp_scale(es < 26u ? 26u : es);
     const float scale_b = seq_ulp_scale(es + 1u < 26u ? 26u : es + 1u);
     uint64_t base = first + (uint64_t)blk * kSeqTile + (uint64_t)threadIdx.x * 16;
-    const bool fresh = PACK && pos + blk >= fresh_from;
+    bool fresh = PACK && pos + blk >= fresh_from;
+    constexpr int NW = kBlock / 64;
+    // ---- whole blocks first try the streaming form ---------------------------------------------
+    // Unless one of its 4096 terms is an exact tie, a block's map is the saturated sum of all its
+    // roundings, however the elements are dealt to the threads (seqsum_core.h).  So the loads are
+    // the coalesced ones of a copy - thread t takes the float4s t, t + 256, t + 512, t + 768 of the
+    // block, non-temporally: every cache line is fetched by one instruction and read once - the
+    // wave adds its sums up by DPP, and only a block that does hold a tie (or an exponent below 26,
+    // where terms are split in integer arithmetic) is done again in order, below.  Packing does not
+    // depend on the order of the sums: four neighbouring lanes hold the four bytes of a word.
+    const uint64_t blk_first = first + (uint64_t)blk * kSeqTile;
+    bool in_order = blk_first + kSeqTile > n || es < 26u;  // (the same for the whole workgroup)
+    if (!in_order) {
+        const float4 *x4 = reinterpret_cast<const float4 *>(x + blk_first);
+        float4 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = ld_stream<true>(x4 + j * kBlock + threadIdx.x);
+        float am[16];
+        uint32_t bytes[4] = {0, 0, 0, 0};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float e[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float a = fabsf(e[i]);
+                const bool take = MASK ? (a > thr) : true;
+                am[4 * j + i] = take ? a : 0.0f;
+                if (fresh) {
+                    bytes[j] |= ternary_code(e[i], thr) << (2 * i);
+                    fresh_count += take ? 1u : 0u;
+                }
+            }
+        }
+        if (fresh) {
+            const int lane = threadIdx.x & 63;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int w = (int)(bytes[j] << (8 * (lane & 3)));
+                w |= __builtin_amdgcn_update_dpp(0, w, 0xB1, 0xf, 0xf, true);  // quad_perm:[1,0,3,2]
+                w |= __builtin_amdgcn_update_dpp(0, w, 0x4E, 0xf, 0xf, true);  // quad_perm:[2,3,0,1]
+                if ((lane & 3) == 0) packed[(blk_first >> 4) + j * (kBlock / 4) + (threadIdx.x >> 2)] = (uint32_t)w;
+            }
+            fresh = false;  // (a second pass over this block packs nothing)
+        }
+        bool tie_a = false, tie_b = false;
+        uint32_t sum_a = seq_min_u32(seq_sum16(am, es, scale, &tie_a), SEQ_SAT), sum_b = 0;
+        if (MULTI) sum_b = seq_min_u32(seq_sum16(am, es + 1u, scale_b, &tie_b), SEQ_SAT);
+        auto wave_add = [](uint32_t u) {  // <= 2^25 per lane: a wave's total stays at or below 2^31
+            int sum = (int)u;
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x111, 0xf, 0xf, true);  // row_shr:1
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x112, 0xf, 0xf, true);  // row_shr:2
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x114, 0xf, 0xf, true);  // row_shr:4
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x118, 0xf, 0xf, true);  // row_shr:8
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x142, 0xa, 0xf, true);  // row_bcast15
+            sum += __builtin_amdgcn_update_dpp(0, sum, 0x143, 0xc, 0xf, true);  // row_bcast31
+            return seq_min_u32((uint32_t)sum, SEQ_SAT);  // lane 63 holds the wave's
+        };
+        sum_a = wave_add(sum_a);
+        if (MULTI) sum_b = wave_add(sum_b);
+        const bool wave_tie = __ballot(tie_a || tie_b) != 0ull;
+        if ((threadIdx.x & 63) == 63) {
+            SeqMap t;
+            t.d0 = sum_a;
+            t.d1 = sum_b | (wave_tie ? 0x80000000u : 0u);  // (sums stay below 2^26)
+            s_wave[threadIdx.x >> 6] = t;
+        }
+        __syncthreads();
+        uint32_t tot_a = 0, tot_b = 0, any_tie = 0;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            const SeqMap t = s_wave[w];
+            tot_a += t.d0;
+            tot_b += t.d1 & 0x7fffffffu;
+            any_tie |= t.d1 & 0x80000000u;
+        }
+        in_order = any_tie != 0;
+        if (!in_order && threadIdx.x == 0) {
+            tot_a = seq_min_u32(tot_a, SEQ_SAT);
+            tot_b = seq_min_u32(tot_b, SEQ_SAT);
+            if (MULTI) {
+                reinterpret_cast<uint4 *>(maps)[blk] = make_uint4(tot_a, tot_a, tot_b, tot_b);
+            } else {
+                SeqMap t;
+                t.d0 = t.d1 = tot_a;
+                maps[blk] = t;
+            }
+        }
+        __syncthreads();  // s_wave is rewritten by the next block, or below
+        if (!in_order) continue;
+    }
+    // ---- in order: a thread's sixteen consecutive elements, the wave's maps composed left to right
     uint32_t word = 0;
     float am[16];  // |x| of the elements that count, +0.0 (the identity as a term) for the others
     if (base + 16 <= n) {
@@ -354,7 +444,6 @@ __device__ __forceinline__ void seq_block_maps_body(
     };
     m = wave_fold(m);
     if (MULTI) mb = wave_fold(mb);
-    constexpr int NW = kBlock / 64;
     if ((threadIdx.x & 63) == 63) {
         s_wave[threadIdx.x >> 6] = m;
         if (MULTI) s_wave[NW + (threadIdx.x >> 6)] = mb;
@@ -387,7 +476,9 @@ __device__ __forceinline__ void seq_block_maps_body(
     }
 }
 
-__global__ __launch_bounds__(kBlock) void seq_block_maps_kernel(
+// (seven waves per SIMD: left to itself the compiler takes 83 registers for the two forms of the body,
+// five waves per SIMD, and the long windows lose what the streaming loads gain)
+__global__ __launch_bounds__(kBlock, 7) void seq_block_maps_kernel(
     const float *__restrict__ x, uint64_t n, int use_mask, float thr,
     const SeqState *__restrict__ state, SeqMap *__restrict__ maps, uint32_t *__restrict__ packed,
     unsigned long long *__restrict__ count_parts) {

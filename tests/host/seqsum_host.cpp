@@ -320,6 +320,56 @@ extern "C" uint64_t seqsum_compare_map16(uint64_t count, uint64_t seed, uint64_t
     return bad;
 }
 
+// A whole block as the maps kernel's streaming form computes it (elements dealt to the threads as a
+// copy would deal them, every thread's sixteen roundings summed, the sums added up) against the
+// ordered form (block_map), on `count` pseudo-random blocks of 4096 terms around the state's ulp.
+// The streaming form is only used when no term is a tie; returns the number of blocks in which it
+// would have been used and disagrees, and in *used how many blocks it would have been used for.
+extern "C" uint64_t seqsum_compare_block_forms(uint64_t count, uint64_t seed, uint64_t *used) {
+    uint64_t bad = 0, fast = 0, x = seed * 0x9E3779B97F4A7C15ull + 1;
+    auto next = [&]() {
+        x ^= x << 13;
+        x ^= x >> 7;
+        x ^= x << 17;
+        return x;
+    };
+    std::vector<float> blk(kTile);
+    for (uint64_t g = 0; g < count; ++g) {
+        const uint32_t es = 26u + (uint32_t)(next() % 200u);
+        const bool short_mantissas = next() % 4u == 0;  // ties happen in these blocks
+        for (int i = 0; i < kTile; ++i) {
+            // ulp/8 .. 512 ulp: the lower bits of such a term are exactly 1000...0 once in 2^3 .. 2^14 draws,
+            // so some blocks hold a tie and most do not
+            uint32_t ex = es - 26u + (uint32_t)(next() % 13u);
+            uint32_t frac = (uint32_t)(next() & 0x7fffffu);
+            if (short_mantissas && next() % 64u == 0) frac &= 0x600000u;
+            if (next() % 5u == 0) { ex = 0; frac = 0; }
+            const uint32_t bits = (ex << 23) | frac;
+            std::memcpy(&blk[i], &bits, 4);
+        }
+        const float scale = seq_ulp_scale(es);
+        uint64_t total = 0;
+        bool any_tie = false;
+        for (int t = 0; t < 256; ++t) {
+            float a[16];
+            for (int j = 0; j < 4; ++j)
+                for (int i = 0; i < 4; ++i) a[4 * j + i] = blk[4 * (j * 256 + t) + i];
+            bool tie;
+            const uint32_t sum = seq_sum16(a, es, scale, &tie);
+            any_tie = any_tie || tie;
+            total += seq_min_u32(sum, SEQ_SAT);
+        }
+        if (any_tie) continue;
+        ++fast;
+        const uint32_t d = total > SEQ_SAT ? SEQ_SAT : (uint32_t)total;
+        const SeqMap want = block_map(blk.data(), 0, kTile, es, 0, 0.0f);
+        const bool w_over = want.d0 >= SEQ_K_LIMIT / 2 || want.d1 >= SEQ_K_LIMIT / 2;
+        if (w_over ? d < SEQ_K_LIMIT / 2 : (want.d0 != d || want.d1 != d)) ++bad;
+    }
+    if (used) *used = fast;
+    return bad;
+}
+
 // Compares the floating-point term split (seq_append_abs, es >= 26) with the integer one
 // (seq_append) on `count` pseudo-random (map, term, exponent) triples.  Returns the number
 // of disagreements: below the limit the maps must be identical; at or above it both must

@@ -119,6 +119,8 @@ def seqsum(tmp_path_factory):
     L.seqsum_literal.argtypes = [C.c_void_p, C.c_uint64, C.c_int, C.c_float]
     L.seqsum_compare_term_splits.restype = C.c_uint64
     L.seqsum_compare_term_splits.argtypes = [C.c_uint64, C.c_uint64]
+    L.seqsum_compare_block_forms.restype = C.c_uint64
+    L.seqsum_compare_block_forms.argtypes = [C.c_uint64, C.c_uint64, C.POINTER(C.c_uint64)]
     L.seqsum_compare_map16.restype = C.c_uint64
     L.seqsum_compare_map16.argtypes = [C.c_uint64, C.c_uint64, C.POINTER(C.c_uint64)]
     return L
@@ -178,6 +180,13 @@ def test_map_of_sixteen_terms_equals_term_by_term(seqsum):
     ties = C.c_uint64()
     assert seqsum.seqsum_compare_map16(400_000, 5, C.byref(ties)) == 0
     assert 1000 < ties.value < 399_000      # both branches were taken
+
+
+def test_a_block_without_ties_is_the_sum_of_its_roundings_in_any_order(seqsum):
+    # the maps kernel's streaming form (coalesced loads, plain sums) against the ordered composition
+    used = C.c_uint64()
+    assert seqsum.seqsum_compare_block_forms(600, 9, C.byref(used)) == 0
+    assert 100 < used.value < 600           # blocks with and without ties were drawn
 
 
 def test_sequential_sum_traffic_is_bounded(seqsum):

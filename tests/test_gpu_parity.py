@@ -123,6 +123,34 @@ def test_strict_abs_sum_when_the_growth_prediction_fails(ctx, n):
     assert cnt_m == surv.size and bits(got_m) == bits(np.cumsum(surv, dtype=np.float32)[-1])
 
 
+@pytest.mark.parametrize("case", range(8))
+def test_quantize_strict_on_random_piecewise_tensors(ctx, case):
+    """Threshold, scale, survivor count and every packed byte of the strict quantiser against numpy's
+    own f32 left folds, on tensors whose scale jumps by orders of magnitude at random places (zero
+    stretches and short mantissas - exact ties - among them)."""
+    rng = np.random.default_rng(1000 + case)
+    n = int(rng.integers(1, 9_000_000)) if case % 2 else int(rng.integers(1, 600_000))
+    x = rng.standard_normal(n).astype(np.float32)
+    cuts = np.concatenate([[0], np.sort(rng.integers(0, n + 1, size=int(rng.integers(0, 9)))), [n]])
+    for a, b in zip(cuts[:-1], cuts[1:]):
+        x[a:b] *= np.float32(0.0 if rng.random() < 0.15 else 10.0 ** rng.uniform(-7, 4))
+    if case % 4 == 0:
+        x = (np.round(x * 64) / 64).astype(np.float32)
+    d_p, packed, scale, thr, survivors = device_quantize(ctx, x)
+    ax = np.abs(x)
+    total = np.cumsum(ax, dtype=np.float32)[-1]
+    thr_want = np.float32(np.float32(total / np.float32(n)) * np.float32(0.7))   # quantization.rs:79
+    assert bits(thr) == bits(thr_want)
+    sv = ax[ax > thr_want]
+    assert survivors == sv.size
+    if sv.size:
+        assert bits(scale) == bits(np.float32(np.cumsum(sv, dtype=np.float32)[-1] / np.float32(sv.size)))
+    codes = np.where(ax <= thr_want, 1, np.where(x > 0, 2, 0)).astype(np.uint8)
+    codes = np.concatenate([codes, np.zeros((-n) % 4, np.uint8)]).reshape(-1, 4)
+    want = (codes[:, 0] | (codes[:, 1] << 2) | (codes[:, 2] << 4) | (codes[:, 3] << 6)).astype(np.uint8)
+    assert (packed == want).all()
+
+
 def test_strict_abs_sum_nonfinite(ctx):
     x = synth_normal(9, 1.0, (100000,))
     for edit, want in (({5000: np.inf}, np.inf), ({5000: np.inf, 90000: np.nan}, np.nan),

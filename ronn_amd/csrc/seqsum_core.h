@@ -261,8 +261,10 @@ SEQ_HD uint32_t seq_multi_rate_lo(double rate) {
 // The next window: its size, and in *multi whether it carries two maps per block.
 SEQ_HD uint64_t seq_plan_window(uint64_t pos, uint64_t total_blocks, double s_now, double rate, uint32_t *multi) {
     if (pos > 0u && pos < SEQ_MULTI_LIMIT && isfinite(s_now)) {
-        uint64_t win = 255u * pos + 64u;  // the second window already measures the growth over hundreds of blocks
-        if (win > SEQ_MULTI_LIMIT - pos) win = SEQ_MULTI_LIMIT - pos;
+        // all the way to the limit: the growth measured over the first block alone is good to a few per
+        // cent for terms of similar size, well inside what the pair of exponents allows (a window of a
+        // few hundred blocks in between, to measure it better, cost a pair of launches for nothing)
+        uint64_t win = SEQ_MULTI_LIMIT - pos;
         if (win > total_blocks - pos) win = total_blocks - pos;
         *multi = 1u;
         return win;

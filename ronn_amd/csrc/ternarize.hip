@@ -1160,11 +1160,11 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     // sizes the next one by the binades S still has to climb (a window ends where S leaves
     // its binade).
     const unsigned grid = (unsigned)(total_blocks < (uint64_t)kMapGrid ? total_blocks : (uint64_t)kMapGrid);
-    // first batch: the binades of the first SEQ_MULTI_LIMIT blocks take three windows (the first
-    // block, and two that carry a pair of maps per block); after them S of similar terms climbs one
+    // first batch: the binades of the first SEQ_MULTI_LIMIT blocks take two windows (the first
+    // block, and one that carries a pair of maps per block); after them S of similar terms climbs one
     // binade per doubling of the position; plus one more (a window that ends early, or a spare
     // pair of launches returns at once: 4 us; another look by the host costs 10-25 us)
-    int batch = 5;
+    int batch = 4;
     RBN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(seq_scan_replay_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSeqScanLds));
     for (uint64_t b = total_blocks / SEQ_MULTI_LIMIT; b > 1; b >>= 1) ++batch;

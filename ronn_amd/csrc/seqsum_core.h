@@ -260,6 +260,10 @@ SEQ_HD uint32_t seq_multi_rate_lo(double rate) {
 
 // The next window: its size, and in *multi whether it carries two maps per block.
 SEQ_HD uint64_t seq_plan_window(uint64_t pos, uint64_t total_blocks, double s_now, double rate, uint32_t *multi) {
+    if (pos == 0u) {  // S = +0 has no binade to make maps for: the first block is resolved on its own
+        *multi = 0u;
+        return 1u;
+    }
     if (pos > 0u && pos < SEQ_MULTI_LIMIT && isfinite(s_now)) {
         // all the way to the limit: the growth measured over the first block alone is good to a few per
         // cent for terms of similar size, well inside what the pair of exponents allows (a window of a

@@ -571,7 +571,9 @@ __device__ __forceinline__ SeqMap seq_block_before(SeqMap m, SeqMap *s_w, SeqMap
 __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x, uint64_t n, uint64_t block_base,
                                                      int use_mask, float thr, uint32_t es, uint32_t k_cur,
                                                      SeqMap *s_w, unsigned *s_first, uint32_t *s_bits_now,
-                                                     float *s_head /* 128 floats */) {
+                                                     float *s_head /* 128 floats */,
+                                                     uint32_t *__restrict__ packed = nullptr /* pack this block too */,
+                                                     unsigned *s_survivors = nullptr /* LDS, zeroed: += its survivors */) {
     const uint32_t t = threadIdx.x;
     constexpr int NW = kBlock / 64;
     const bool worker = __builtin_amdgcn_readfirstlane((int)(t >> 6)) < NW;  // wave-uniform
@@ -606,19 +608,34 @@ __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x
     }
     const uint64_t base = block_base + (uint64_t)t * 16;
     float a[16];
+    uint32_t word = 0;  // the thread's sixteen elements as one packed word (only when packing)
     if (base + 16 <= n && (reinterpret_cast<uintptr_t>(x + base) & 15u) == 0) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const float4 v = reinterpret_cast<const float4 *>(x + base)[j];
             a[4 * j] = fabsf(v.x), a[4 * j + 1] = fabsf(v.y), a[4 * j + 2] = fabsf(v.z), a[4 * j + 3] = fabsf(v.w);
+            if (packed)
+                word |= (ternary_code(v.x, thr) | ternary_code(v.y, thr) << 2 | ternary_code(v.z, thr) << 4 |
+                         ternary_code(v.w, thr) << 6) << (8 * j);
         }
     } else {
 #pragma unroll
         for (int i = 0; i < 16; ++i) a[i] = 0.0f;
         for (int i = 0; i < 16; ++i) {
             const uint64_t idx = base + i;
-            if (idx < n) a[i] = fabsf(x[idx]);
+            if (idx < n) {
+                const float v = x[idx];
+                a[i] = fabsf(v);
+                if (packed) word |= ternary_code(v, thr) << (2 * i);
+            }
         }
+    }
+    if (packed) {
+        if (base < n) packed[base >> 4] = word;  // tail bits stay zero
+        unsigned mine = 0;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mine += a[i] > thr ? 1u : 0u;  // (elements past the end are +0.0; a NaN is no survivor)
+        if (mine) atomicAdd(s_survivors, mine);
     }
     // a skipped element adds +0.0, which leaves any S >= 0 (and NaN/Inf) unchanged, and as a
     // term of a map it is the identity
@@ -746,8 +763,8 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     const SeqMap *__restrict__ maps, const float *__restrict__ x, uint64_t n, uint64_t total_blocks,
     int use_mask, float thr, SeqState *__restrict__ state, SeqState *__restrict__ host_copy,
     int mirror /* the last launch of a batch: the host reads the state after it */,
-    const unsigned long long *__restrict__ count_parts /* packing sums: the maps kernels' survivor counters */,
-    int n_parts) {
+    unsigned long long *__restrict__ count_parts /* packing sums: the maps kernels' survivor counters */,
+    int n_parts, uint32_t *__restrict__ packed /* packing sums: the packed words (the first block is packed here) */) {
     extern __shared__ uint4 s_maps[];  // SEQ_MULTI_LIMIT units: the maps of a window with two per block
     __shared__ SeqMap s_w[16];
     __shared__ unsigned s_first;
@@ -756,6 +773,7 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     __shared__ unsigned long long s_min64;
     __shared__ uint32_t s_edge[64];
     __shared__ unsigned long long s_cnt64[16];
+    __shared__ unsigned s_cnt0;
     __shared__ __attribute__((aligned(16))) float s_head[128];
     const uint32_t t = threadIdx.x;
     // Windows of up to 1024 blocks (most of them) have one map per thread: it is requested
@@ -816,6 +834,21 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         *state = next;
         if (mirror) *host_copy = next;  // a store to pinned host memory: only when somebody will look
     };
+
+    // ---- the first block of a sum: S = +0 has no binade to make maps for; the block is replayed at
+    // once (no maps launch runs before this one), and packed here when the sum goes with packing
+    if (pos0 == 0 && bits0 == 0u && nblocks == 1u) {
+        if (t == 0) s_cnt0 = 0;
+        __syncthreads();
+        const uint32_t result_bits = seq_replay_block(x, n, 0, use_mask, thr, 1u, 0u, s_w, &s_first, &s_bits_now, s_head,
+                                                      count_parts ? packed : nullptr, &s_cnt0);
+        __syncthreads();
+        if (t == 0 && count_parts) count_parts[n_parts - 1] = s_cnt0;  // the last slot is this block's
+        __syncthreads();
+        count_survivors(1);
+        if (t == 0) finish(result_bits, 1);
+        return;
+    }
 
     // ---- a window with two maps per block: through as many binades as the maps hold ---------
     if (state->multi) {
@@ -1146,7 +1179,7 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     // at least 1024 map slots: the window-end kernel reads slot threadIdx.x before it knows the window
     // and two per block for the windows that span several binades
     const uint64_t map_slots = total_blocks > 2 * SEQ_MULTI_LIMIT ? total_blocks : 2 * SEQ_MULTI_LIMIT;
-    RBN_CHECK(rbn_workspace(ctx, kScratchHeader + map_slots * sizeof(SeqMap) + kMapGrid * 8, &ws));
+    RBN_CHECK(rbn_workspace(ctx, kScratchHeader + map_slots * sizeof(SeqMap) + (kMapGrid + 1) * 8, &ws));
     ReduceScratch *scr = (ReduceScratch *)ws;
     SeqMap *maps = (SeqMap *)((char *)ws + kScratchHeader);
     unsigned long long *count_parts =
@@ -1154,7 +1187,7 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     SeqState *h_state = (SeqState *)ctx->mailbox;
     memset(h_state, 0, sizeof(SeqState));
     seq_init_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(
-        &scr->seq, (uint32_t)seq_next_window(0, total_blocks, 0.0, 0.0), count_parts, kMapGrid);
+        &scr->seq, 1u /* the first window is the first block */, count_parts, kMapGrid + 1);
     // Windows are queued in batches: the kernels take each window from the device state and
     // return at once when the sum is complete, so the host only looks in between batches and
     // sizes the next one by the binades S still has to climb (a window ends where S leaves
@@ -1168,19 +1201,24 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     RBN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(seq_scan_replay_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSeqScanLds));
     for (uint64_t b = total_blocks / SEQ_MULTI_LIMIT; b > 1; b >>= 1) ++batch;
+    bool first_batch = true;
     for (;;) {
         for (int i = 0; i < batch; ++i) {
-            seq_block_maps_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
-                d_x, n, use_mask, thr, &scr->seq, maps, (uint32_t *)d_packed, count_parts);
+            // (the very first window is the first block from S = +0: the window-end kernel replays it
+            // without maps, so no maps launch goes before it)
+            if (!(first_batch && i == 0))
+                seq_block_maps_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
+                    d_x, n, use_mask, thr, &scr->seq, maps, (uint32_t *)d_packed, count_parts);
             seq_scan_replay_kernel<<<dim3(1), dim3(1024), kSeqScanLds, ctx->stream>>>(
                 maps, d_x, n, total_blocks, use_mask, thr, &scr->seq, h_state, i == batch - 1, count_parts,
-                (int)grid);
+                kMapGrid + 1, (uint32_t *)d_packed);
         }
         RBN_HIP(hipGetLastError());
         RBN_HIP(hipStreamSynchronize(ctx->stream));
         if (h_state->error)
             return rbn_fail(RBN_ERR_HIP, "sequential-sum scan made no progress (internal error)");
         if (h_state->done) break;
+        first_batch = false;
         float s_now;
         memcpy(&s_now, &h_state->s_bits, 4);
         // S grows by about s_now * (blocks left / blocks done) more: one window per doubling

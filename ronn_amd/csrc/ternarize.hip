@@ -272,13 +272,13 @@ __device__ __forceinline__ SeqMap seq_dpp(SeqMap m) {
 template <bool MULTI, bool MASK, bool PACK>
 __device__ __forceinline__ void seq_block_maps_body(
     const float *__restrict__ x, uint64_t n, float thr,
-    const SeqState *__restrict__ state, SeqMap *__restrict__ maps, uint32_t *__restrict__ packed,
+    const SeqState &st, SeqMap *__restrict__ maps, uint32_t *__restrict__ packed,
     unsigned long long *__restrict__ count_parts, SeqMap *s_wave, unsigned *s_cnt) {
-    const uint32_t win = state->win;
-    const uint64_t fresh_from = state->fresh_from, pos = state->pos;
+    const uint32_t win = st.win;
+    const uint64_t fresh_from = st.fresh_from, pos = st.pos;
     unsigned fresh_count = 0;
-    const uint64_t first = state->pos * kSeqTile;
-    const uint32_t s_bits = state->s_bits, rate_lo = state->rate_lo;
+    const uint64_t first = st.pos * kSeqTile;
+    const uint32_t s_bits = st.s_bits, rate_lo = st.rate_lo;
     uint32_t es0, k_unused;
     seq_state_split(s_bits, &es0, &k_unused);
   for (uint32_t blk = blockIdx.x; blk < win; blk += gridDim.x) {
@@ -303,6 +303,9 @@ __device__ __forceinline__ void seq_block_maps_body(
         float4 v[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = ld_stream<true>(x4 + j * kBlock + threadIdx.x);
+        // (all four loads go out before the first value is touched: short of registers, the compiler
+        // had put the first load's wait and use between the first and the second load)
+        __builtin_amdgcn_sched_barrier(0);
         float am[16];
         uint32_t bytes[4] = {0, 0, 0, 0};
 #pragma unroll
@@ -383,6 +386,7 @@ __device__ __forceinline__ void seq_block_maps_body(
         float4 v[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) v[j] = reinterpret_cast<const float4 *>(x + base)[j];
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             float e[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
@@ -484,19 +488,25 @@ __global__ __launch_bounds__(kBlock, 7) void seq_block_maps_kernel(
     unsigned long long *__restrict__ count_parts) {
     __shared__ SeqMap s_wave[2 * (kBlock / 64)];
     __shared__ unsigned s_cnt[kBlock / 64];
-    if (state->done) return;
-    // (plain loads also in long windows: a thread's four loads share their cache lines, and
-    // non-temporal ones fetched each line four times - 98 -> 130 us for the last window of 8192 x 28672)
+    // the whole state in one scalar round trip (asked for field by field, `done`, `multi` and the
+    // window each cost a dependent one before the first load of data could go out)
+    asm volatile("" : : "s"(x), "s"(n), "s"(use_mask), "s"(thr), "s"(state), "s"(maps), "s"(packed), "s"(count_parts));
+    const SeqState st = *state;
+    asm volatile("" : : "s"(st.s_bits), "s"(st.win), "s"(st.pos), "s"(st.done), "s"(st.multi), "s"(st.fresh_from),
+                 "s"(st.rate_lo));
+    if (st.done) return;
+    // (in the ordered form plain loads also in long windows: a thread's four loads share their cache
+    // lines, and non-temporal ones fetched each line four times)
     auto run = [&](auto multi) {
         constexpr bool M = decltype(multi)::value;
         if (packed != nullptr)  // packing goes with a masked sum (thr is the ternary threshold)
-            seq_block_maps_body<M, true, true>(x, n, thr, state, maps, packed, count_parts, s_wave, s_cnt);
+            seq_block_maps_body<M, true, true>(x, n, thr, st, maps, packed, count_parts, s_wave, s_cnt);
         else if (use_mask)
-            seq_block_maps_body<M, true, false>(x, n, thr, state, maps, packed, count_parts, s_wave, s_cnt);
+            seq_block_maps_body<M, true, false>(x, n, thr, st, maps, packed, count_parts, s_wave, s_cnt);
         else
-            seq_block_maps_body<M, false, false>(x, n, thr, state, maps, packed, count_parts, s_wave, s_cnt);
+            seq_block_maps_body<M, false, false>(x, n, thr, st, maps, packed, count_parts, s_wave, s_cnt);
     };
-    if (state->multi)
+    if (st.multi)
         run(std::true_type{});
     else
         run(std::false_type{});

@@ -790,17 +790,21 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     // here, before the state is known, so that the two round trips overlap (the buffer holds
     // at least 1024 maps).
     const SeqMap spec = maps[t];
-    const uint32_t done0 = state->done;
-    // (both values are named here so that both loads are issued before either is waited for)
-    asm volatile("" : : "v"(spec.d0), "v"(spec.d1), "s"(done0));
+    // the whole state in the same round trip (field by field, `done`, the window, `multi` and its
+    // rate each cost a dependent one)
+    const SeqState st0 = *state;
+    // (all values are named here so that every load is issued before any is waited for)
+    asm volatile("" : : "v"(spec.d0), "v"(spec.d1), "s"(st0.done), "s"(st0.win), "s"(st0.pos), "s"(st0.s_bits),
+                 "s"(st0.multi), "s"(st0.rate_lo), "s"(st0.fresh_from));
+    const uint32_t done0 = st0.done;
     if (done0) {
         if (mirror && t == 0) *host_copy = *state;
         return;
     }
-    const uint32_t nblocks = state->win;
-    const uint64_t pos0 = state->pos;
+    const uint32_t nblocks = st0.win;
+    const uint64_t pos0 = st0.pos;
     const uint64_t first = pos0 * kSeqTile;
-    const uint32_t bits0 = state->s_bits;
+    const uint32_t bits0 = st0.s_bits;
     uint32_t es, k0;
     seq_state_split(bits0, &es, &k0);
     // ends the window: the state after `advanced` blocks, the next window's size from the
@@ -839,7 +843,7 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         next.saw_nan = 0;
         next.pad = 0;
         next.survivors = survivors_total;
-        const uint64_t seen = pos0 + nblocks, before = state->fresh_from;
+        const uint64_t seen = pos0 + nblocks, before = st0.fresh_from;
         next.fresh_from = seen > before ? seen : before;
         *state = next;
         if (mirror) *host_copy = next;  // a store to pinned host memory: only when somebody will look
@@ -861,10 +865,10 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     }
 
     // ---- a window with two maps per block: through as many binades as the maps hold ---------
-    if (state->multi) {
+    if (st0.multi) {
         // at most SEQ_MULTI_LIMIT blocks: eight per thread, loaded once (both maps of a block are
         // one 16-byte load)
-        const uint32_t rate_lo = state->rate_lo;
+        const uint32_t rate_lo = st0.rate_lo;
         if (nblocks > SEQ_MULTI_LIMIT) {  // not a window the plan makes: reported as an internal error
             if (t == 0) finish(bits0, 0);
             return;

@@ -581,15 +581,15 @@ __device__ __forceinline__ SeqMap seq_block_before(SeqMap m, SeqMap *s_w, SeqMap
 __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x, uint64_t n, uint64_t block_base,
                                                      int use_mask, float thr, uint32_t es, uint32_t k_cur,
                                                      SeqMap *s_w, unsigned *s_first, uint32_t *s_bits_now,
-                                                     float *s_head /* 128 floats */,
+                                                     float *s_head /* 512 floats */,
                                                      uint32_t *__restrict__ packed = nullptr /* pack this block too */,
                                                      unsigned *s_survivors = nullptr /* LDS, zeroed: += its survivors */) {
     const uint32_t t = threadIdx.x;
     constexpr int NW = kBlock / 64;
     const bool worker = __builtin_amdgcn_readfirstlane((int)(t >> 6)) < NW;  // wave-uniform
     // A sum that starts at zero doubles every few elements: crossed binade by binade, the first
-    // 128 elements cost seven turns of the loop below.  They are added one after the other instead
-    // (that IS the fold, so it is exact whatever the state).
+    // 512 elements cost nine turns of the loop below.  They are added one after the other instead
+    // (that IS the fold, so it is exact whatever the state; 2 us for the 512 additions).
     const bool head = es == 1u && k_cur == 0u;
     if (!worker) {
         // the barriers of the worker waves, in the same order, and their exits
@@ -655,7 +655,7 @@ __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x
     uint32_t done = 0;  // chunks [0, done) are already folded into (es, k_cur)
     uint32_t result_bits = 0;
     if (head) {
-        constexpr uint32_t kHeadChunks = 8;
+        constexpr uint32_t kHeadChunks = 32;
         if (t < kHeadChunks) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) s_head[t * 16 + i] = a[i];
@@ -784,7 +784,7 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     __shared__ uint32_t s_edge[64];
     __shared__ unsigned long long s_cnt64[16];
     __shared__ unsigned s_cnt0;
-    __shared__ __attribute__((aligned(16))) float s_head[128];
+    __shared__ __attribute__((aligned(16))) float s_head[512];
     const uint32_t t = threadIdx.x;
     // Windows of up to 1024 blocks (most of them) have one map per thread: it is requested
     // here, before the state is known, so that the two round trips overlap (the buffer holds

@@ -245,7 +245,7 @@ struct SeqState {
     uint32_t multi;     // the window carries two maps per block (seq_plan_window)
     uint64_t fresh_from;  // blocks from here on have not been seen by any window yet
     uint32_t rate_lo;   // multi: the cautious growth of S per block (f32 bits) behind the blocks' exponents
-    uint32_t pad;
+    uint32_t thr_bits;  // a sum queued behind another one: its mask threshold (f32 bits), set on the device
     uint64_t survivors;  // packing sums only: elements above the threshold, set by the window that ends the sum
 };
 
@@ -483,18 +483,20 @@ __device__ __forceinline__ void seq_block_maps_body(
 // (seven waves per SIMD: left to itself the compiler takes 83 registers for the two forms of the body,
 // five waves per SIMD, and the long windows lose what the streaming loads gain)
 __global__ __launch_bounds__(kBlock, 7) void seq_block_maps_kernel(
-    const float *__restrict__ x, uint64_t n, int use_mask, float thr,
+    const float *__restrict__ x, uint64_t n, int use_mask, float thr_arg, int thr_from_state,
     const SeqState *__restrict__ state, SeqMap *__restrict__ maps, uint32_t *__restrict__ packed,
     unsigned long long *__restrict__ count_parts) {
     __shared__ SeqMap s_wave[2 * (kBlock / 64)];
     __shared__ unsigned s_cnt[kBlock / 64];
     // the whole state in one scalar round trip (asked for field by field, `done`, `multi` and the
     // window each cost a dependent one before the first load of data could go out)
-    asm volatile("" : : "s"(x), "s"(n), "s"(use_mask), "s"(thr), "s"(state), "s"(maps), "s"(packed), "s"(count_parts));
+    asm volatile("" : : "s"(x), "s"(n), "s"(use_mask), "s"(thr_arg), "s"(state), "s"(maps), "s"(packed),
+                 "s"(count_parts));
     const SeqState st = *state;
     asm volatile("" : : "s"(st.s_bits), "s"(st.win), "s"(st.pos), "s"(st.done), "s"(st.multi), "s"(st.fresh_from),
                  "s"(st.rate_lo));
     if (st.done) return;
+    const float thr = thr_from_state ? __uint_as_float(st.thr_bits) : thr_arg;
     // (in the ordered form plain loads also in long windows: a thread's four loads share their cache
     // lines, and non-temporal ones fetched each line four times)
     auto run = [&](auto multi) {
@@ -521,7 +523,31 @@ __global__ __launch_bounds__(kBlock) void seq_init_kernel(SeqState *__restrict__
     if (threadIdx.x == 0) {
         SeqState z;
         z.s_bits = 0, z.win = win0, z.pos = 0, z.done = 0, z.error = 0, z.saw_nan = 0, z.multi = 0;
-        z.fresh_from = 0, z.rate_lo = 0, z.pad = 0, z.survivors = 0;
+        z.fresh_from = 0, z.rate_lo = 0, z.thr_bits = 0, z.survivors = 0;
+        *state = z;
+    }
+}
+
+// The state of a sum that is queued behind another one without the host in between: the masked sum
+// of the quantiser, whose threshold is (S / n) * 0.7 of the sum before it (quantization.rs:79).  If
+// that sum is not complete when this kernel runs (its batch of windows was too short, or S left the
+// finite range), the follower is marked done with error 2: its kernels return at once and the host
+// runs it the ordinary way afterwards.
+__global__ __launch_bounds__(kBlock) void seq_chain_init_kernel(const SeqState *__restrict__ prev,
+                                                               SeqState *__restrict__ state, uint64_t n,
+                                                               uint64_t total_blocks,
+                                                               unsigned long long *__restrict__ count_parts,
+                                                               int n_parts) {
+    if (count_parts)
+        for (int i = threadIdx.x; i < n_parts; i += kBlock) count_parts[i] = 0;
+    if (threadIdx.x == 0) {
+        const SeqState p = *prev;
+        const bool complete = p.done && !p.error && p.pos >= total_blocks && ((p.s_bits >> 23) & 0xffu) != 0xffu;
+        SeqState z;
+        z.s_bits = 0, z.win = 1u, z.pos = 0, z.done = complete ? 0u : 1u, z.error = complete ? 0u : 2u;
+        z.saw_nan = 0, z.multi = 0, z.fresh_from = 0, z.rate_lo = 0, z.survivors = 0;
+        const float mean = __uint_as_float(p.s_bits) / (float)n;
+        z.thr_bits = __float_as_uint(mean * 0.7f);
         *state = z;
     }
 }
@@ -771,7 +797,7 @@ __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x
 // host mailbox (the host reads it after synchronising: it sizes the next window).
 __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     const SeqMap *__restrict__ maps, const float *__restrict__ x, uint64_t n, uint64_t total_blocks,
-    int use_mask, float thr, SeqState *__restrict__ state, SeqState *__restrict__ host_copy,
+    int use_mask, float thr_arg, int thr_from_state, SeqState *__restrict__ state, SeqState *__restrict__ host_copy,
     int mirror /* the last launch of a batch: the host reads the state after it */,
     unsigned long long *__restrict__ count_parts /* packing sums: the maps kernels' survivor counters */,
     int n_parts, uint32_t *__restrict__ packed /* packing sums: the packed words (the first block is packed here) */) {
@@ -801,6 +827,7 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         if (mirror && t == 0) *host_copy = *state;
         return;
     }
+    const float thr = thr_from_state ? __uint_as_float(st0.thr_bits) : thr_arg;
     const uint32_t nblocks = st0.win;
     const uint64_t pos0 = st0.pos;
     const uint64_t first = pos0 * kSeqTile;
@@ -841,7 +868,7 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         next.multi = next.done ? 0u : next_multi;
         next.rate_lo = seq_multi_rate_lo(rate);
         next.saw_nan = 0;
-        next.pad = 0;
+        next.thr_bits = st0.thr_bits;
         next.survivors = survivors_total;
         const uint64_t seen = pos0 + nblocks, before = st0.fresh_from;
         next.fresh_from = seen > before ? seen : before;
@@ -1161,6 +1188,7 @@ __global__ __launch_bounds__(kBlock) void tile_weights_kernel(
 // Device scalars used by the reductions, at the start of the context workspace.
 struct ReduceScratch {
     SeqState seq;
+    SeqState seq_next;  // the sum queued behind `seq`
     unsigned long long survivors;
     float tree_sum;
     uint32_t pad0;
@@ -1178,10 +1206,33 @@ constexpr size_t kSeqScanLds = (size_t)SEQ_MULTI_LIMIT * 16;  // dynamic LDS of 
 int pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold, uint8_t *d_packed,
                  uint64_t *h_survivors, float *h_survivor_sum);
 
+// One sum as the window kernels see it.
+struct SeqRun {
+    int use_mask;
+    float thr;
+    int thr_from_state;  // the kernels take the threshold from the device state instead of thr
+    SeqState *d_state, *h_state;
+    uint32_t *d_packed;
+    unsigned long long *count_parts;
+};
+
+// A second sum queued behind the first without the host in between: the quantiser's masked sum,
+// whose threshold (S / n) * 0.7 the device derives from the first sum's result.  `ran` is false
+// when the chain broke (the first sum needed another look by the host, or left the finite range):
+// the caller then runs the second sum the ordinary way.
+struct SeqFollower {
+    uint8_t *d_packed;
+    float *h_sum;
+    uint64_t *h_survivors;
+    bool ran;
+};
+
 // With d_packed given (use_mask must be set, thr is the ternary threshold) the same pass also
 // packs the tensor and counts the survivors into *h_survivors.
 int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, float thr,
-                   float *h_sum, uint8_t *d_packed = nullptr, uint64_t *h_survivors = nullptr) {
+                   float *h_sum, uint8_t *d_packed = nullptr, uint64_t *h_survivors = nullptr,
+                   SeqFollower *follower = nullptr) {
+    if (follower) follower->ran = false;
     if (n == 0) {
         *h_sum = -0.0f;  // Rust's empty f32 sum
         if (h_survivors) *h_survivors = 0;
@@ -1196,52 +1247,67 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     RBN_CHECK(rbn_workspace(ctx, kScratchHeader + map_slots * sizeof(SeqMap) + (kMapGrid + 1) * 8, &ws));
     ReduceScratch *scr = (ReduceScratch *)ws;
     SeqMap *maps = (SeqMap *)((char *)ws + kScratchHeader);
-    unsigned long long *count_parts =
-        d_packed ? (unsigned long long *)((char *)ws + kScratchHeader + map_slots * sizeof(SeqMap)) : nullptr;
-    SeqState *h_state = (SeqState *)ctx->mailbox;
-    memset(h_state, 0, sizeof(SeqState));
+    unsigned long long *parts_mem = (unsigned long long *)((char *)ws + kScratchHeader + map_slots * sizeof(SeqMap));
+    SeqRun main_run{use_mask, thr, 0, &scr->seq, (SeqState *)ctx->mailbox, (uint32_t *)d_packed,
+                    d_packed ? parts_mem : nullptr};
+    memset(main_run.h_state, 0, sizeof(SeqState));
     seq_init_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(
-        &scr->seq, 1u /* the first window is the first block */, count_parts, kMapGrid + 1);
+        main_run.d_state, 1u /* the first window is the first block */, main_run.count_parts, kMapGrid + 1);
     // Windows are queued in batches: the kernels take each window from the device state and
     // return at once when the sum is complete, so the host only looks in between batches and
     // sizes the next one by the binades S still has to climb (a window ends where S leaves
     // its binade).
     const unsigned grid = (unsigned)(total_blocks < (uint64_t)kMapGrid ? total_blocks : (uint64_t)kMapGrid);
-    // first batch: the binades of the first SEQ_MULTI_LIMIT blocks take two windows (the first
-    // block, and one that carries a pair of maps per block); after them S of similar terms climbs one
-    // binade per doubling of the position; plus one more (a window that ends early, or a spare
-    // pair of launches returns at once: 4 us; another look by the host costs 10-25 us)
-    int batch = 4;
     RBN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(seq_scan_replay_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSeqScanLds));
-    for (uint64_t b = total_blocks / SEQ_MULTI_LIMIT; b > 1; b >>= 1) ++batch;
-    bool first_batch = true;
-    for (;;) {
+    auto queue_batch = [&](const SeqRun &r, int batch, bool first_batch) {
         for (int i = 0; i < batch; ++i) {
             // (the very first window is the first block from S = +0: the window-end kernel replays it
             // without maps, so no maps launch goes before it)
             if (!(first_batch && i == 0))
                 seq_block_maps_kernel<<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
-                    d_x, n, use_mask, thr, &scr->seq, maps, (uint32_t *)d_packed, count_parts);
+                    d_x, n, r.use_mask, r.thr, r.thr_from_state, r.d_state, maps, r.d_packed, r.count_parts);
             seq_scan_replay_kernel<<<dim3(1), dim3(1024), kSeqScanLds, ctx->stream>>>(
-                maps, d_x, n, total_blocks, use_mask, thr, &scr->seq, h_state, i == batch - 1, count_parts,
-                kMapGrid + 1, (uint32_t *)d_packed);
+                maps, d_x, n, total_blocks, r.use_mask, r.thr, r.thr_from_state, r.d_state, r.h_state,
+                i == batch - 1, r.count_parts, kMapGrid + 1, r.d_packed);
         }
-        RBN_HIP(hipGetLastError());
-        RBN_HIP(hipStreamSynchronize(ctx->stream));
-        if (h_state->error)
-            return rbn_fail(RBN_ERR_HIP, "sequential-sum scan made no progress (internal error)");
-        if (h_state->done) break;
-        first_batch = false;
-        float s_now;
-        memcpy(&s_now, &h_state->s_bits, 4);
-        // S grows by about s_now * (blocks left / blocks done) more: one window per doubling
-        const double done_blocks = (double)h_state->pos, left = (double)(total_blocks - h_state->pos);
-        const double growth = 1.0 + left / (done_blocks > 1.0 ? done_blocks : 1.0);
-        batch = (int)(log2(growth) + 1.5);
-        batch = batch < 1 ? 1 : (batch > 16 ? 16 : batch);
-        (void)s_now;
+    };
+    // Looks at the state the last batch left and queues batches until the sum is complete.
+    auto run_to_end = [&](const SeqRun &r) -> int {
+        for (;;) {
+            if (r.h_state->error)
+                return rbn_fail(RBN_ERR_HIP, "sequential-sum scan made no progress (internal error)");
+            if (r.h_state->done) return RBN_OK;
+            // S grows by about s_now * (blocks left / blocks done) more: one window per doubling
+            const double done_blocks = (double)r.h_state->pos, left = (double)(total_blocks - r.h_state->pos);
+            const double growth = 1.0 + left / (done_blocks > 1.0 ? done_blocks : 1.0);
+            int batch = (int)(log2(growth) + 1.5);
+            batch = batch < 1 ? 1 : (batch > 16 ? 16 : batch);
+            queue_batch(r, batch, false);
+            RBN_HIP(hipGetLastError());
+            RBN_HIP(hipStreamSynchronize(ctx->stream));
+        }
+    };
+    // first batch: the binades of the first SEQ_MULTI_LIMIT blocks take two windows (the first
+    // block, and one that carries a pair of maps per block); after them S of similar terms climbs one
+    // binade per doubling of the position; plus one more (a window that ends early, or a spare
+    // pair of launches returns at once: 4 us; another look by the host costs 10-25 us)
+    int batch = 4;
+    for (uint64_t b = total_blocks / SEQ_MULTI_LIMIT; b > 1; b >>= 1) ++batch;
+    queue_batch(main_run, batch, true);
+    SeqRun next_run{};
+    if (follower) {
+        next_run = SeqRun{1, 0.0f, 1, &scr->seq_next, (SeqState *)((char *)ctx->mailbox + 256),
+                          (uint32_t *)follower->d_packed, parts_mem};
+        memset(next_run.h_state, 0, sizeof(SeqState));
+        seq_chain_init_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(
+            main_run.d_state, next_run.d_state, n, total_blocks, next_run.count_parts, kMapGrid + 1);
+        queue_batch(next_run, batch, true);
     }
+    RBN_HIP(hipGetLastError());
+    RBN_HIP(hipStreamSynchronize(ctx->stream));
+    RBN_CHECK(run_to_end(main_run));
+    SeqState *h_state = main_run.h_state;
     const uint32_t s_bits = h_state->s_bits;
     const uint64_t pos = h_state->pos;
     float s;
@@ -1264,6 +1330,28 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
             RBN_CHECK(pack_ternary(ctx, d_x, n, thr, d_packed, h_survivors, nullptr));
         } else if (h_survivors) {
             *h_survivors = h_state->survivors;  // added up by the window that folded the last block
+        }
+    }
+    if (follower) {
+        SeqState *h_next = next_run.h_state;
+        // the threshold the device derived must be the host's own (same two IEEE operations)
+        volatile float mean = s / (float)n;
+        volatile float host_thr = mean * 0.7f;
+        float thr_f = host_thr;
+        uint32_t host_thr_bits;
+        memcpy(&host_thr_bits, &thr_f, 4);
+        const bool chained = !(h_next->done && h_next->error == 2u) && h_next->thr_bits == host_thr_bits &&
+                             is_finite_bits(s_bits) && pos >= total_blocks;
+        if (chained) {
+            RBN_CHECK(run_to_end(next_run));
+            float s_next;
+            memcpy(&s_next, &h_next->s_bits, 4);
+            *follower->h_sum = s_next;
+            if (h_next->pos < total_blocks)
+                RBN_CHECK(pack_ternary(ctx, d_x, n, thr_f, follower->d_packed, follower->h_survivors, nullptr));
+            else
+                *follower->h_survivors = h_next->survivors;
+            follower->ran = true;
         }
     }
     return RBN_OK;
@@ -1397,19 +1485,19 @@ int rbn_quantize_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, int mode, u
     }
     // quantization.rs:79: (sum / n as f32) * 0.7
     float sum = 0.0f;
-    if (mode == RBN_SUM_TREE)
-        RBN_CHECK(tree_abs_sum(ctx, d_x, n, 0, 0.0f, &sum, nullptr));
-    else
-        RBN_CHECK(strict_abs_sum(ctx, d_x, n, 0, 0.0f, &sum));
+    if (mode == RBN_SUM_TREE) RBN_CHECK(tree_abs_sum(ctx, d_x, n, 0, 0.0f, &sum, nullptr));
+    uint64_t survivors = 0;
+    float nz_sum = 0.0f;
+    SeqFollower masked{d_packed, &nz_sum, &survivors, false};
+    if (mode != RBN_SUM_TREE)
+        RBN_CHECK(strict_abs_sum(ctx, d_x, n, 0, 0.0f, &sum, nullptr, nullptr, &masked));
     volatile float mean = sum / (float)n;
     volatile float threshold = mean * 0.7f;
     // quantization.rs:100 (pack) and the survivor count of :82-91
     // (one pass in either mode: the survivors' sum, their count and the packed words)
-    uint64_t survivors = 0;
-    float nz_sum = 0.0f;
     if (mode == RBN_SUM_TREE)
         RBN_CHECK(pack_ternary(ctx, d_x, n, threshold, d_packed, &survivors, &nz_sum));
-    else
+    else if (!masked.ran)
         RBN_CHECK(strict_abs_sum(ctx, d_x, n, 1, threshold, &nz_sum, d_packed, &survivors));
     // quantization.rs:93-97
     float scale = 1.0f;

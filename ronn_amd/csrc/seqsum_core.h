@@ -36,6 +36,7 @@
 
 #define SEQ_K_LIMIT (1u << 24)  // k >= this: S has left the binade
 #define SEQ_SAT (1u << 25)      // saturation value of d0/d1
+#define SEQ_BLOCK_ELEMS 4096u   // elements per block map
 
 struct SeqMap {
     uint32_t d0;  // increment of k when the incoming k is even
@@ -203,26 +204,68 @@ SEQ_HD SeqMap seq_compose(SeqMap a, SeqMap b) {
 // Applies a map to a concrete k.
 SEQ_HD uint32_t seq_apply(SeqMap m, uint32_t k) { return k + ((k & 1u) ? m.d1 : m.d0); }
 
-// ---- host-side window policy -------------------------------------------------------------
+// ---- window policy ---------------------------------------------------------------------------
 // The block maps of a window are valid for one binade, so a window should end where S is
-// expected to leave it.  `s_now` is the current sum, `rate` its recent growth per block
-// (<= 0: unknown).  Without a rate the window is half again what has been summed so far
-// (S of similar terms doubles when the position doubles); with one, the distance to the
-// binade's upper edge at that rate plus a margin.  When growth slows down (rounding eats
-// more of every term in a higher binade) the window just ends early and the next one
-// continues with a fresh rate; blocks past a crossing are the only wasted reads.
+// expected to leave it.  `s_now` is the current sum, `rate` its growth per block (<= 0: unknown)
+// measured over `rate_elems` elements.  The growth differs from binade to binade (in a higher one
+// rounding eats more of every term, up to all of it), so the rate that counts is the one since S
+// entered its present binade: the window-end kernel measures it from the last crossing on, be it
+// over the rest of the crossing block only.  Without a rate the window is half again what has been
+// summed so far (S of similar terms doubles when the position doubles); with one, the distance to
+// the binade's upper edge at that rate plus a margin of 10 % and of 2.5 standard errors of a mean of
+// `rate_elems` half-normal terms (0.75 / sqrt(m) each).  A window that ends short of the crossing
+// costs a pair of launches (12 us); the blocks past a crossing are the only wasted reads (2.5 ns
+// each).
 #include <math.h>
-SEQ_HD uint64_t seq_next_window(uint64_t pos, uint64_t total_blocks, double s_now, double rate) {
+SEQ_HD uint64_t seq_next_window(uint64_t pos, uint64_t total_blocks, double s_now, double rate, double rate_elems) {
     uint64_t win = pos + pos / 2;
     if (rate > 0.0 && s_now > 0.0 && isfinite(s_now)) {
         int e = 0;
         (void)frexp(s_now, &e);  // s_now = m * 2^e, m in [0.5, 1): the binade ends at 2^e
         const double need = (ldexp(1.0, e) - s_now) / rate;
-        win = need < 1e15 ? (uint64_t)(need * 1.10) + 4u : total_blocks;
+        const double margin = 1.10 + (rate_elems >= 1.0 && rate_elems < 1e8 ? 1.9 / sqrt(rate_elems) : 0.0);
+        win = need < 1e15 ? (uint64_t)(need * margin) + 4u : total_blocks;
     }
     if (win < 64u) win = 64u;
     if (win > total_blocks - pos) win = total_blocks - pos;
     return win;
+}
+
+// The growth per block that sizes the next window, from what a window saw: S before and after it,
+// the blocks it folded, S right behind its last crossing (s_before when there was none) and the
+// blocks folded since (a fraction when the window ended inside the crossing block).  Fewer than 64
+// elements behind the crossing say too little: then the average over the window stands in.  The
+// first window of a sum (s_before = 0) always takes its average: S climbs through its first
+// binades inside one block, at one rate.
+SEQ_HD double seq_window_rate(double s_before, double s_after, double advanced, double s_cross, double since_cross,
+                              double *rate_elems) {
+    double rate = advanced > 0.0 ? (s_after - s_before) / advanced : 0.0;
+    *rate_elems = advanced * (double)SEQ_BLOCK_ELEMS;
+    if (s_before > 0.0 && since_cross * (double)SEQ_BLOCK_ELEMS >= 64.0 && since_cross <= advanced) {
+        rate = (s_after - s_cross) / since_cross;
+        *rate_elems = since_cross * (double)SEQ_BLOCK_ELEMS;
+    }
+    return rate;
+}
+
+// ---- where a window's block maps lie -------------------------------------------------------------
+// The window-end kernel gives each of its 1024 threads a run of consecutive blocks: `chunk` =
+// ceil(win / 1024) of them up to 32, and longer windows in stretches of 32768 blocks, 32 per thread.
+// The maps are stored transposed to that: the i-th block of thread t's run lies at slot
+// i * 1024 + t (of its stretch), so that what the 64 lanes of a wave load together is contiguous
+// (with the maps in block order every lane asked for a cache line of its own, and one compute unit
+// took 10 us for 32768 maps).  Slots stay below win rounded up to 1024, or to 32768 in stretches.
+#define SEQ_SCAN_THREADS 1024u
+#define SEQ_SCAN_RUN 32u  // the longest run of blocks per thread
+SEQ_HD uint32_t seq_map_slot(uint32_t block, uint32_t win) {
+    if (win <= SEQ_SCAN_THREADS) return block;
+    const uint32_t stretch_blocks = SEQ_SCAN_THREADS * SEQ_SCAN_RUN;
+    if (win <= stretch_blocks) {
+        const uint32_t chunk = (win + SEQ_SCAN_THREADS - 1u) / SEQ_SCAN_THREADS;
+        return (block % chunk) * SEQ_SCAN_THREADS + block / chunk;
+    }
+    const uint32_t r = block % stretch_blocks;
+    return (block - r) + (r % SEQ_SCAN_RUN) * SEQ_SCAN_THREADS + r / SEQ_SCAN_RUN;
 }
 
 // ---- windows that span several binades ------------------------------------------------------
@@ -259,7 +302,8 @@ SEQ_HD uint32_t seq_multi_rate_lo(double rate) {
 }
 
 // The next window: its size, and in *multi whether it carries two maps per block.
-SEQ_HD uint64_t seq_plan_window(uint64_t pos, uint64_t total_blocks, double s_now, double rate, uint32_t *multi) {
+SEQ_HD uint64_t seq_plan_window(uint64_t pos, uint64_t total_blocks, double s_now, double rate, double rate_elems,
+                                uint32_t *multi) {
     if (pos == 0u) {  // S = +0 has no binade to make maps for: the first block is resolved on its own
         *multi = 0u;
         return 1u;
@@ -274,7 +318,7 @@ SEQ_HD uint64_t seq_plan_window(uint64_t pos, uint64_t total_blocks, double s_no
         return win;
     }
     *multi = 0u;
-    return seq_next_window(pos, total_blocks, s_now, rate);
+    return seq_next_window(pos, total_blocks, s_now, rate, rate_elems);
 }
 
 #endif  // RONN_SEQSUM_CORE_H

@@ -31,6 +31,7 @@ constexpr uint64_t kStreamBytes = 192ull << 20;  // tensors above this size are 
 
 constexpr int kBlock = 256;
 constexpr int kSeqTile = 4096;  // elements per block map of the sequential sum (256 x 16)
+static_assert(kSeqTile == (int)SEQ_BLOCK_ELEMS, "the window policy counts elements per block");
 
 __device__ __forceinline__ uint32_t ternary_code(float v, float threshold) {
     // quantization.rs:138-144.  NaN fails both comparisons and packs as 00 (-1).
@@ -373,7 +374,7 @@ __device__ __forceinline__ void seq_block_maps_body(
             } else {
                 SeqMap t;
                 t.d0 = t.d1 = tot_a;
-                maps[blk] = t;
+                maps[seq_map_slot(blk, win)] = t;
             }
         }
         __syncthreads();  // s_wave is rewritten by the next block, or below
@@ -461,7 +462,7 @@ __device__ __forceinline__ void seq_block_maps_body(
             for (int w = 1; w < NW; ++w) u = seq_compose(u, s_wave[NW + w]);
             reinterpret_cast<uint4 *>(maps)[blk] = make_uint4(t.d0, t.d1, u.d0, u.d1);
         } else {
-            maps[blk] = t;
+            maps[seq_map_slot(blk, win)] = t;
         }
     }
     __syncthreads();  // s_wave is rewritten in the next turn
@@ -608,6 +609,8 @@ __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x
                                                      int use_mask, float thr, uint32_t es, uint32_t k_cur,
                                                      SeqMap *s_w, unsigned *s_first, uint32_t *s_bits_now,
                                                      float *s_head /* 512 floats */,
+                                                     uint32_t *s_cross /* [0]: S behind the block's last crossing
+                                                                          chunk, [1]: chunks folded up to there */,
                                                      uint32_t *__restrict__ packed = nullptr /* pack this block too */,
                                                      unsigned *s_survivors = nullptr /* LDS, zeroed: += its survivors */) {
     const uint32_t t = threadIdx.x;
@@ -680,6 +683,7 @@ __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x
     const int lane = t & 63, wave = t >> 6;
     uint32_t done = 0;  // chunks [0, done) are already folded into (es, k_cur)
     uint32_t result_bits = 0;
+    uint32_t cross_bits = seq_state_join(es, k_cur), cross_done = 0;  // the last crossing so far: none
     if (head) {
         constexpr uint32_t kHeadChunks = 32;
         if (t < kHeadChunks) {
@@ -713,6 +717,7 @@ __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x
             return *s_bits_now;  // (already in LDS for the other waves)
         }
         seq_state_split(result_bits, &es, &k_cur);
+        cross_bits = result_bits, cross_done = done;
     }
     for (int guard = 0; guard <= kBlock; ++guard) {
         SeqMap m = seq_identity();
@@ -756,6 +761,7 @@ __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x
         __syncthreads();  // (3)
         result_bits = *s_bits_now;
         done = tstar + 1;
+        cross_bits = result_bits, cross_done = done;
         if (((result_bits >> 23) & 0xffu) == 0xffu) {
             // S is +Inf or NaN.  +Inf turns into NaN if a NaN follows inside this block.
             bool nan_after = false;
@@ -777,7 +783,10 @@ __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x
     // barrier before reading it).  The store cannot overtake a read: with no crossing in this turn
     // nobody has read s_bits_now since the last turn's barrier (3), two barriers ago; on the other
     // exits it holds this very value already.
-    if (t == 0) *s_bits_now = result_bits;
+    if (t == 0) {
+        *s_bits_now = result_bits;
+        s_cross[0] = cross_bits, s_cross[1] = cross_done;  // (read by thread 0 only, or behind the caller's barrier)
+    }
     return result_bits;
 }
 
@@ -811,6 +820,7 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     __shared__ unsigned long long s_cnt64[16];
     __shared__ unsigned s_cnt0;
     __shared__ __attribute__((aligned(16))) float s_head[512];
+    __shared__ uint32_t s_cross[2];
     const uint32_t t = threadIdx.x;
     // Windows of up to 1024 blocks (most of them) have one map per thread: it is requested
     // here, before the state is known, so that the two round trips overlap (the buffer holds
@@ -853,18 +863,22 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
             survivors_total = sum;
         }
     };
-    auto finish = [&](uint32_t bits, uint32_t advanced) {
+    // (cross_bits: S right behind the window's last crossing, since_cross: the blocks folded since, a
+    // fraction inside the crossing block; bits0 and `advanced` for a window without a crossing)
+    auto finish = [&](uint32_t bits, uint32_t advanced, uint32_t cross_bits, double since_cross) {
         const uint64_t pos = pos0 + advanced;
         const bool finite = ((bits >> 23) & 0xffu) != 0xffu;
         const double s_before = (double)__uint_as_float(bits0), s_after = (double)__uint_as_float(bits);
-        const double rate = advanced ? (s_after - s_before) / (double)advanced : 0.0;
+        double rate_elems = 0.0;
+        const double rate = seq_window_rate(s_before, s_after, (double)advanced, (double)__uint_as_float(cross_bits),
+                                            since_cross, &rate_elems);
         SeqState next;
         next.s_bits = bits;
         next.pos = pos;
         next.error = (advanced == 0 || advanced > nblocks) ? 1u : 0u;
         next.done = (pos >= total_blocks || !finite || next.error) ? 1u : 0u;
         uint32_t next_multi = 0u;
-        next.win = next.done ? 0u : (uint32_t)seq_plan_window(pos, total_blocks, s_after, rate, &next_multi);
+        next.win = next.done ? 0u : (uint32_t)seq_plan_window(pos, total_blocks, s_after, rate, rate_elems, &next_multi);
         next.multi = next.done ? 0u : next_multi;
         next.rate_lo = seq_multi_rate_lo(rate);
         next.saw_nan = 0;
@@ -882,12 +896,12 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         if (t == 0) s_cnt0 = 0;
         __syncthreads();
         const uint32_t result_bits = seq_replay_block(x, n, 0, use_mask, thr, 1u, 0u, s_w, &s_first, &s_bits_now, s_head,
-                                                      count_parts ? packed : nullptr, &s_cnt0);
+                                                      s_cross, count_parts ? packed : nullptr, &s_cnt0);
         __syncthreads();
         if (t == 0 && count_parts) count_parts[n_parts - 1] = s_cnt0;  // the last slot is this block's
         __syncthreads();
         count_survivors(1);
-        if (t == 0) finish(result_bits, 1);
+        if (t == 0) finish(result_bits, 1, bits0, 1.0);
         return;
     }
 
@@ -897,7 +911,7 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         // one 16-byte load)
         const uint32_t rate_lo = st0.rate_lo;
         if (nblocks > SEQ_MULTI_LIMIT) {  // not a window the plan makes: reported as an internal error
-            if (t == 0) finish(bits0, 0);
+            if (t == 0) finish(bits0, 0, bits0, 0.0);
             return;
         }
         // The window's maps go to LDS once (both maps of a block are one 16-byte unit): kept in
@@ -935,6 +949,8 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         }
         __syncthreads();
         uint32_t b_cur = 0, cur_bits = bits0;
+        uint32_t cross_bits = bits0, cross_block = 0, cross_chunks = 0;  // the last crossing
+        bool crossed = false;
         for (int guard = 0; guard < 48; ++guard) {
             uint32_t k_in;
             seq_state_split(cur_bits, &es, &k_in);
@@ -985,28 +1001,38 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
             }
             const uint32_t cb = (uint32_t)(first_cross >> 32), k_cb = (uint32_t)first_cross;
             (void)seq_replay_block(x, n, first + (uint64_t)cb * kSeqTile, use_mask, thr, es, k_cb, s_w, &s_first,
-                                   &s_bits_now, s_head);
+                                   &s_bits_now, s_head, s_cross);
             __syncthreads();  // the result is in LDS; s_w and s_min64 are rewritten in the next turn
             cur_bits = s_bits_now;
+            cross_bits = s_cross[0], cross_chunks = s_cross[1], cross_block = cb, crossed = true;
             b_cur = cb + 1u;
             if (((cur_bits >> 23) & 0xffu) == 0xffu || b_cur >= nblocks) break;
         }
         count_survivors(b_cur);
-        if (t == 0) finish(cur_bits, b_cur);
+        // blocks folded since the last crossing: the rest of its block and the whole ones behind it
+        const double since = !crossed
+                                 ? (double)b_cur
+                                 : (double)(b_cur - cross_block - 1u) + (double)((uint32_t)kBlock - cross_chunks) / kBlock;
+        if (t == 0) finish(cur_bits, b_cur, cross_bits, since);
         return;
     }
 
     // ---- (1) scan -----------------------------------------------------------------------
     {
         const uint32_t chunk = (nblocks + 1023u) / 1024u;
-        const uint32_t lo = t * chunk;
-        const uint32_t hi = lo + chunk < nblocks ? lo + chunk : nblocks;
+        uint32_t lo = t * chunk;
+        uint32_t hi = lo + chunk < nblocks ? lo + chunk : nblocks;
         // A thread's maps are loaded once, all loads in flight, and kept in registers for
-        // both walks (composition, then the search for the crossing) when there are at
-        // most 32 of them (windows up to 32768 blocks); longer chunks are walked twice in
-        // batches of eight.  Spare slots re-read the chunk's last map and are skipped.
+        // both walks (composition, then the search for the crossing): up to 32 of them.  A window of
+        // more than 32768 blocks is walked in stretches of that many, each from the state the one
+        // before it ends in, up to the stretch that holds the crossing (in batches of eight per thread,
+        // one round trip to memory after the other, 45,000 blocks took 36 us; so they take 8).
+        // Spare slots re-read the chunk's last map and are skipped.
         SeqMap mine = seq_identity();
         uint32_t k = 0, cand = 0xffffffffu, cand_k = 0;
+        uint32_t k_in = k0;  // the state that enters the stretch
+        SeqMap stretch = seq_identity();  // the map of the whole stretch
+        const SeqMap *run_maps = maps + t;  // the thread's run: every 1024th slot from here (seq_map_slot)
         if (t == 0) s_first = 0xffffffffu;
         auto walk_cached = [&](auto size_tag) {
             constexpr int C = decltype(size_tag)::value;
@@ -1015,14 +1041,13 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
                 mm[0] = spec;
             } else {
 #pragma unroll
-                for (int i = 0; i < C; ++i) mm[i] = maps[lo + i < hi ? lo + i : (hi > 0 ? hi - 1 : 0)];
+                for (int i = 0; i < C; ++i) mm[i] = run_maps[(uint32_t)i * SEQ_SCAN_THREADS];  // (slots past the run are skipped)
             }
 #pragma unroll
             for (int i = 0; i < C; ++i)
                 if (lo + i < hi) mine = seq_compose(mine, mm[i]);
-            SeqMap all;
-            const SeqMap before = seq_block_before<16>(mine, s_w, &all);
-            k = seq_apply(before, k0);
+            const SeqMap before = seq_block_before<16>(mine, s_w, &stretch);
+            k = seq_apply(before, k_in);
             if (k < SEQ_K_LIMIT) {
 #pragma unroll
                 for (int i = 0; i < C; ++i) {
@@ -1045,35 +1070,20 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         } else if (chunk <= 32u) {
             walk_cached(std::integral_constant<int, 32>{});
         } else {
-            for (uint32_t b0 = lo; b0 < hi; b0 += 8) {
-                SeqMap mm[8];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) mm[i] = maps[b0 + i < hi ? b0 + i : hi - 1];
-#pragma unroll
-                for (int i = 0; i < 8; ++i)
-                    if (b0 + i < hi) mine = seq_compose(mine, mm[i]);
-            }
-            SeqMap all;
-            const SeqMap before = seq_block_before<16>(mine, s_w, &all);
-            k = seq_apply(before, k0);
-            if (k < SEQ_K_LIMIT) {
-                for (uint32_t b0 = lo; b0 < hi && cand == 0xffffffffu; b0 += 8) {
-                    SeqMap mm[8];
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) mm[i] = maps[b0 + i < hi ? b0 + i : hi - 1];
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        if (b0 + i < hi && cand == 0xffffffffu) {
-                            const uint32_t k2 = seq_apply(mm[i], k);
-                            if (k2 >= SEQ_K_LIMIT) {
-                                cand = b0 + i;
-                                cand_k = k;
-                            } else {
-                                k = k2;
-                            }
-                        }
-                    }
-                }
+            constexpr uint32_t kStretch = SEQ_SCAN_THREADS * SEQ_SCAN_RUN;
+            for (uint32_t from = 0; from < nblocks; from += kStretch) {
+                const uint32_t to = nblocks - from > kStretch ? from + kStretch : nblocks;
+                lo = from + t * SEQ_SCAN_RUN;
+                lo = lo < to ? lo : to;
+                hi = lo + SEQ_SCAN_RUN < to ? lo + SEQ_SCAN_RUN : to;
+                run_maps = maps + from + t;
+                mine = seq_identity();
+                walk_cached(std::integral_constant<int, 32>{});
+                if (to == nblocks) break;  // the last stretch: its crossing, or the end of the window, is settled below
+                if (cand != 0xffffffffu) atomicMin(&s_first, cand);
+                __syncthreads();  // (also: s_w is rewritten by the next stretch)
+                if (s_first != 0xffffffffu) break;
+                k_in = seq_apply(stretch, k_in);
             }
         }
         if (cand != 0xffffffffu) atomicMin(&s_first, cand);
@@ -1095,15 +1105,15 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     uint32_t k_cur = s_cross_k;
     if (cb == 0xffffffffu) {
         count_survivors(nblocks);
-        if (t == 0) finish(seq_state_join(es, k_cur), nblocks);
+        if (t == 0) finish(seq_state_join(es, k_cur), nblocks, bits0, (double)nblocks);
         return;
     }
 
     // ---- (2) replay of block cb
     const uint32_t result_bits = seq_replay_block(x, n, first + (uint64_t)cb * kSeqTile, use_mask, thr, es, k_cur,
-                                                  s_w, &s_first, &s_bits_now, s_head);
+                                                  s_w, &s_first, &s_bits_now, s_head, s_cross);
     count_survivors(cb + 1);
-    if (t == 0) finish(result_bits, cb + 1);
+    if (t == 0) finish(result_bits, cb + 1, s_cross[0], (double)((uint32_t)kBlock - s_cross[1]) / kBlock);
 }
 
 __global__ __launch_bounds__(kBlock) void any_nan_kernel(const float *__restrict__ x,
@@ -1243,7 +1253,11 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     void *ws = nullptr;
     // at least 1024 map slots: the window-end kernel reads slot threadIdx.x before it knows the window
     // and two per block for the windows that span several binades
-    const uint64_t map_slots = total_blocks > 2 * SEQ_MULTI_LIMIT ? total_blocks : 2 * SEQ_MULTI_LIMIT;
+    // and a stretch more than blocks: the maps of a window are stored transposed (seq_map_slot), in
+    // slots up to the window rounded up to a stretch, and the window-end kernel loads a thread's
+    // whole run of slots whatever the window
+    const uint64_t map_slots = (total_blocks > 2 * SEQ_MULTI_LIMIT ? total_blocks : 2 * SEQ_MULTI_LIMIT) +
+                               SEQ_SCAN_THREADS * SEQ_SCAN_RUN;
     RBN_CHECK(rbn_workspace(ctx, kScratchHeader + map_slots * sizeof(SeqMap) + (kMapGrid + 1) * 8, &ws));
     ReduceScratch *scr = (ReduceScratch *)ws;
     SeqMap *maps = (SeqMap *)((char *)ws + kScratchHeader);

@@ -62,10 +62,30 @@ struct ScanResult {
     uint32_t k;
 };
 
+ScanResult scan_stretch(const std::vector<SeqMap> &maps, uint32_t from, uint32_t to, uint32_t k0, SeqMap *total);
+
+// The scan of a window: in one piece up to 32768 blocks (32 maps per thread), longer ones in
+// stretches of 32768, each from the state the stretch before it ends in.
 ScanResult scan(const std::vector<SeqMap> &maps, uint32_t s_bits) {
     const uint32_t nblocks = (uint32_t)maps.size();
     uint32_t es, k0;
     seq_state_split(s_bits, &es, &k0);
+    SeqMap total;
+    if (nblocks <= 32768u) return scan_stretch(maps, 0, nblocks, k0, &total);
+    uint32_t k_in = k0;
+    for (uint32_t from = 0;; from += 32768u) {
+        const uint32_t to = nblocks - from > 32768u ? from + 32768u : nblocks;
+        ScanResult r = scan_stretch(maps, from, to, k_in, &total);
+        if (r.cross_block != 0xffffffffu || to == nblocks) return r;
+        k_in = seq_apply(total, k_in);
+    }
+}
+
+// Blocks [from, to) of the window from the state k0: the first block in which k reaches 2^24 (as an
+// index into the window) and the k that enters it, or no block and the k after the last one.
+ScanResult scan_stretch(const std::vector<SeqMap> &all_maps, uint32_t from, uint32_t to, uint32_t k0, SeqMap *total) {
+    const std::vector<SeqMap> maps(all_maps.begin() + from, all_maps.begin() + to);
+    const uint32_t nblocks = to - from;
     const uint32_t chunk = (nblocks + 1023u) / 1024u;
     std::vector<SeqMap> a(1024), b(1024);
     for (uint32_t t = 0; t < 1024; ++t) {
@@ -107,11 +127,12 @@ ScanResult scan(const std::vector<SeqMap> &maps, uint32_t s_bits) {
     for (uint32_t t = 0; t < 1024; ++t) {
         uint32_t lo = t * chunk, hi = lo + chunk < nblocks ? lo + chunk : nblocks;
         if (first != 0xffffffffu) {
-            if (cand[t] == first) r = ScanResult{first, cand_k[t]};
+            if (cand[t] == first) r = ScanResult{from + first, cand_k[t]};
         } else if (hi == nblocks && lo < hi) {
             r = ScanResult{0xffffffffu, last_k[t]};
         }
     }
+    *total = (*src)[1023];
     return r;
 }
 }  // namespace
@@ -119,8 +140,9 @@ ScanResult scan(const std::vector<SeqMap> &maps, uint32_t s_bits) {
 // The replay of one block (the second half of the window-end kernel): crossings inside the
 // block are resolved one after another.  Returns the state after the block as f32 bits.
 static uint32_t replay_block(const float *x, uint64_t n, uint64_t bbase, int use_mask, float thr,
-                             uint32_t es, uint32_t k_cur) {
+                             uint32_t es, uint32_t k_cur, uint32_t *cross_bits, uint32_t *cross_chunks) {
     uint32_t done = 0, result_bits = 0;
+    *cross_bits = seq_state_join(es, k_cur), *cross_chunks = 0;
     for (int guard = 0; guard <= 256; ++guard) {
         SeqMap cm[256], a[256], b2[256];
         for (int t = 0; t < 256; ++t)
@@ -167,6 +189,7 @@ static uint32_t replay_block(const float *x, uint64_t n, uint64_t bbase, int use
         }
         std::memcpy(&result_bits, &s, 4);
         done = (uint32_t)tstar + 1;
+        *cross_bits = result_bits, *cross_chunks = done;
         if (((result_bits >> 23) & 0xff) == 0xff) {
             for (uint64_t idx = bbase + (uint64_t)done * 16; idx < bbase + kTile && idx < n; ++idx) {
                 bool take = use_mask ? (std::fabs(x[idx]) > thr) : true;
@@ -191,7 +214,7 @@ extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr
     const uint64_t total_blocks = (n + kTile - 1) / kTile;
     uint64_t pos = 0;  // in blocks
     uint32_t s_bits = 0;
-    double rate = 0.0;
+    double rate = 0.0, rate_elems = 0.0;
     while (pos < total_blocks) {
         if (((s_bits >> 23) & 0xff) == 0xff) break;
         uint32_t es0, k0;
@@ -199,7 +222,7 @@ extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr
         float s_before;
         std::memcpy(&s_before, &s_bits, 4);
         uint32_t multi = 0;
-        const uint64_t win = seq_plan_window(pos, total_blocks, (double)s_before, rate, &multi);
+        const uint64_t win = seq_plan_window(pos, total_blocks, (double)s_before, rate, rate_elems, &multi);
         const uint32_t rate_lo = seq_multi_rate_lo(rate);
         const uint32_t nm = multi ? 2u : 1u;
         const uint64_t first = pos * kTile;
@@ -217,6 +240,10 @@ extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr
         // while the blocks' maps hold it
         uint64_t b_cur = 0;
         uint32_t cur_bits = s_bits;
+        // the last crossing of the window: S right behind its chunk, and where it was
+        bool crossed = false;
+        uint32_t cross_bits = s_bits, cross_chunks = 0;
+        uint64_t cross_block = 0;
         for (int guard = 0; guard < 64; ++guard) {
             uint32_t es, k;
             seq_state_split(cur_bits, &es, &k);
@@ -231,7 +258,9 @@ extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr
                 b_cur = range_end;
                 break;
             }
-            cur_bits = replay_block(x, n, first + (b_cur + sr.cross_block) * kTile, use_mask, thr, es, sr.k);
+            cur_bits = replay_block(x, n, first + (b_cur + sr.cross_block) * kTile, use_mask, thr, es, sr.k,
+                                    &cross_bits, &cross_chunks);
+            crossed = true, cross_block = b_cur + sr.cross_block;
             b_cur += (uint64_t)sr.cross_block + 1;
             if (((cur_bits >> 23) & 0xff) == 0xff || b_cur >= win) break;
         }
@@ -239,7 +268,12 @@ extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr
         s_bits = cur_bits;
         float s_after;
         std::memcpy(&s_after, &s_bits, 4);
-        rate = ((double)s_after - (double)s_before) / (double)b_cur;
+        float s_cross;
+        std::memcpy(&s_cross, &cross_bits, 4);
+        const double since = !crossed ? (double)b_cur
+                                      : (double)(b_cur - cross_block - 1) + (double)(256u - cross_chunks) / 256.0;
+        rate = seq_window_rate((double)s_before, (double)s_after, (double)b_cur, (double)s_cross,
+                               since, &rate_elems);
         pos += b_cur;
         ++iters;
     }
@@ -411,5 +445,40 @@ extern "C" uint64_t seqsum_compare_term_splits(uint64_t count, uint64_t seed) {
             ++bad;
         }
     }
+    return bad;
+}
+
+// The transposed storage of a window's maps against the runs the window-end kernel gives its
+// threads: thread t's i-th block must lie at slot i * 1024 + t of its stretch, no two blocks may
+// share a slot, and no slot may lie beyond the window rounded up to a stretch.  Returns the
+// number of violations.
+extern "C" uint64_t seqsum_check_map_slots(uint32_t win) {
+    uint64_t bad = 0;
+    const uint32_t stretch = SEQ_SCAN_THREADS * SEQ_SCAN_RUN;
+    std::vector<uint8_t> taken((size_t)((win + stretch - 1) / stretch) * stretch, 0);
+    auto claim = [&](uint32_t block, uint32_t expect) {
+        const uint32_t slot = seq_map_slot(block, win);
+        if (slot != expect || slot >= taken.size() || taken[slot]) ++bad;
+        if (slot < taken.size()) taken[slot] = 1;
+    };
+    uint32_t seen = 0;
+    if (win <= stretch) {
+        const uint32_t chunk = (win + SEQ_SCAN_THREADS - 1) / SEQ_SCAN_THREADS;
+        for (uint32_t t = 0; t < SEQ_SCAN_THREADS; ++t) {
+            const uint32_t lo = t * chunk, hi = lo + chunk < win ? lo + chunk : win;
+            for (uint32_t b = lo; b < hi; ++b, ++seen) claim(b, (b - lo) * SEQ_SCAN_THREADS + t);
+        }
+    } else {
+        for (uint32_t from = 0; from < win; from += stretch) {
+            const uint32_t to = win - from > stretch ? from + stretch : win;
+            for (uint32_t t = 0; t < SEQ_SCAN_THREADS; ++t) {
+                uint32_t lo = from + t * SEQ_SCAN_RUN;
+                lo = lo < to ? lo : to;
+                const uint32_t hi = lo + SEQ_SCAN_RUN < to ? lo + SEQ_SCAN_RUN : to;
+                for (uint32_t b = lo; b < hi; ++b, ++seen) claim(b, from + (b - lo) * SEQ_SCAN_THREADS + t);
+            }
+        }
+    }
+    if (seen != win) ++bad;
     return bad;
 }

@@ -123,6 +123,27 @@ def test_strict_abs_sum_when_the_growth_prediction_fails(ctx, n):
     assert cnt_m == surv.size and bits(got_m) == bits(np.cumsum(surv, dtype=np.float32)[-1])
 
 
+def test_strict_abs_sum_with_a_crossing_deep_inside_a_long_window(ctx):
+    """One term of 1.0 per block of 4096 behind a first term of 2^16: S climbs one unit per block, the
+    window that follows block 8192 is some 63,000 blocks long, and S leaves its binade (at 2^17) beyond
+    block 57,000 of that window - in the second of the stretches of 32,768 maps the window-end kernel
+    walks.  Every partial sum is an integer below 2^24, so the fold is exact and its value known."""
+    blocks = 72_000
+    n = blocks * 4096
+    x = np.zeros(n, dtype=np.float32)
+    x[5::4096] = -1.0
+    x[0] = 65536.0
+    want = np.float32(65536 + blocks)
+    d_x = ctx.to_device(x)
+    got, cnt = ctx.abs_sum(d_x, n, STRICT)
+    assert bits(got) == bits(want) and cnt == n
+    got_m, cnt_m = ctx.abs_sum(d_x, n, STRICT, mask_threshold=np.float32(0.75))
+    assert bits(got_m) == bits(want) and cnt_m == blocks + 1
+    got_1, cnt_1 = ctx.abs_sum(d_x, n, STRICT, mask_threshold=np.float32(2.0))
+    assert bits(got_1) == bits(np.float32(65536)) and cnt_1 == 1
+    d_x.free()
+
+
 @pytest.mark.parametrize("case", range(8))
 def test_quantize_strict_on_random_piecewise_tensors(ctx, case):
     """Threshold, scale, survivor count and every packed byte of the strict quantiser against numpy's

@@ -123,6 +123,8 @@ def seqsum(tmp_path_factory):
     L.seqsum_compare_block_forms.argtypes = [C.c_uint64, C.c_uint64, C.POINTER(C.c_uint64)]
     L.seqsum_compare_map16.restype = C.c_uint64
     L.seqsum_compare_map16.argtypes = [C.c_uint64, C.c_uint64, C.POINTER(C.c_uint64)]
+    L.seqsum_check_map_slots.restype = C.c_uint64
+    L.seqsum_check_map_slots.argtypes = [C.c_uint32]
     return L
 
 
@@ -167,6 +169,25 @@ def test_parallel_sequential_sum_is_bit_exact(seqsum, name, x):
         want = np.float32(seqsum.seqsum_literal(x.ctypes.data, x.size, mask, thr))
         assert got.view(np.uint32) == want.view(np.uint32) or (np.isnan(got) and np.isnan(want)), \
             "%s mask=%d: %r vs %r" % (name, mask, got, want)
+
+
+def test_transposed_map_slots_match_the_runs_of_the_window_end_kernel(seqsum):
+    # every block of a window at slot i * 1024 + t of its thread's run, one block per slot, inside the buffer
+    for win in (1, 2, 1023, 1024, 1025, 2047, 2048, 2049, 4565, 8192, 8193, 32767, 32768, 32769, 45005,
+                65535, 65536, 65537, 100_000, 1_000_003):
+        assert seqsum.seqsum_check_map_slots(win) == 0, win
+
+
+def test_a_window_longer_than_one_stretch_is_walked_stretch_by_stretch(seqsum):
+    # one term of 1.0 per block behind a first term of 2^16: the window behind block 8192 is 63,000 blocks
+    # long and S leaves its binade beyond block 57,000 of it (second stretch of 32,768 maps); all sums exact
+    blocks = 72_000
+    x = np.zeros(blocks * 4096, dtype=np.float32)
+    x[5::4096] = -1.0
+    x[0] = 65536.0
+    it = C.c_uint64()
+    got = np.float32(seqsum.seqsum_host(x.ctypes.data, x.size, 0, 0.0, C.byref(it), None))
+    assert got == np.float32(65536 + blocks) and it.value == 5
 
 
 def test_float_and_integer_term_splits_agree(seqsum):

@@ -38,6 +38,8 @@ struct rbn_ctx {
     // One word of RBN_FLAG_* bits that kernels set when they refuse to do something a host
     // check could not see coming (rbn_device_flags reads and clears it).
     unsigned *dev_flags = nullptr;
+    // the window-end kernel of the exact sums has been given its dynamic-LDS limit on this device
+    bool seq_scan_prepared = false;
 };
 
 constexpr int RBN_SPLITK_TILES = 16384;  // 64 MiB

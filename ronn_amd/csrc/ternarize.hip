@@ -1262,6 +1262,11 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     ReduceScratch *scr = (ReduceScratch *)ws;
     SeqMap *maps = (SeqMap *)((char *)ws + kScratchHeader);
     unsigned long long *parts_mem = (unsigned long long *)((char *)ws + kScratchHeader + map_slots * sizeof(SeqMap));
+    if (!ctx->seq_scan_prepared) {  // (once per context: the call costs the host a few microseconds)
+        RBN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(seq_scan_replay_kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSeqScanLds));
+        ctx->seq_scan_prepared = true;
+    }
     SeqRun main_run{use_mask, thr, 0, &scr->seq, (SeqState *)ctx->mailbox, (uint32_t *)d_packed,
                     d_packed ? parts_mem : nullptr};
     memset(main_run.h_state, 0, sizeof(SeqState));
@@ -1272,8 +1277,6 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     // sizes the next one by the binades S still has to climb (a window ends where S leaves
     // its binade).
     const unsigned grid = (unsigned)(total_blocks < (uint64_t)kMapGrid ? total_blocks : (uint64_t)kMapGrid);
-    RBN_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(seq_scan_replay_kernel),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSeqScanLds));
     auto queue_batch = [&](const SeqRun &r, int batch, bool first_batch) {
         for (int i = 0; i < batch; ++i) {
             // (the very first window is the first block from S = +0: the window-end kernel replays it

@@ -556,6 +556,32 @@ __global__ __launch_bounds__(kBlock) void seq_chain_init_kernel(const SeqState *
     }
 }
 
+// Inclusive ordered scan of a wave's maps (lane l ends with the composition of lanes 0..l).  Maps that
+// do not depend on the parity of k - all of them unless a term was an exact tie - are plain
+// increments, and composing increments is adding them and saturating once at the end (the sum of 64
+// saturated increments stays below 2^31): one DPP add per step instead of a composition of ten
+// instructions.  The choice is made per wave, so all lanes take the same path.
+__device__ __forceinline__ SeqMap seq_wave_inclusive(SeqMap m) {
+    if (__ballot(m.d0 != m.d1) == 0ull) {
+        int sum = (int)m.d0;
+        sum += __builtin_amdgcn_update_dpp(0, sum, 0x111, 0xf, 0xf, true);  // row_shr:1
+        sum += __builtin_amdgcn_update_dpp(0, sum, 0x112, 0xf, 0xf, true);  // row_shr:2
+        sum += __builtin_amdgcn_update_dpp(0, sum, 0x114, 0xf, 0xf, true);  // row_shr:4
+        sum += __builtin_amdgcn_update_dpp(0, sum, 0x118, 0xf, 0xf, true);  // row_shr:8
+        sum += __builtin_amdgcn_update_dpp(0, sum, 0x142, 0xa, 0xf, true);  // row_bcast15: rows 1, 3 absorb the row before
+        sum += __builtin_amdgcn_update_dpp(0, sum, 0x143, 0xc, 0xf, true);  // row_bcast31: rows 2, 3 absorb rows 0-1
+        m.d0 = m.d1 = seq_min_u32((uint32_t)sum, SEQ_SAT);
+        return m;
+    }
+    m = seq_compose(seq_dpp<0x111, 0xf>(m), m);  // row_shr:1
+    m = seq_compose(seq_dpp<0x112, 0xf>(m), m);  // row_shr:2
+    m = seq_compose(seq_dpp<0x114, 0xf>(m), m);  // row_shr:4
+    m = seq_compose(seq_dpp<0x118, 0xf>(m), m);  // row_shr:8
+    m = seq_compose(seq_dpp<0x142, 0xa>(m), m);  // row_bcast15
+    m = seq_compose(seq_dpp<0x143, 0xc>(m), m);  // row_bcast31
+    return m;
+}
+
 // Ordered scans of SeqMaps without a barrier per step: inside a wave by shuffles (lane l
 // absorbs what lies to its left), across the waves through one LDS slot per wave.  Returns the
 // composition of everything BEFORE this thread, and in *total the composition of all; NW = waves
@@ -565,12 +591,7 @@ template <int NW>
 __device__ __forceinline__ SeqMap seq_block_before(SeqMap m, SeqMap *s_w, SeqMap *total) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     // inclusive scan of the wave: inside rows of 16 lanes, then across the rows
-    m = seq_compose(seq_dpp<0x111, 0xf>(m), m);  // row_shr:1
-    m = seq_compose(seq_dpp<0x112, 0xf>(m), m);  // row_shr:2
-    m = seq_compose(seq_dpp<0x114, 0xf>(m), m);  // row_shr:4
-    m = seq_compose(seq_dpp<0x118, 0xf>(m), m);  // row_shr:8
-    m = seq_compose(seq_dpp<0x142, 0xa>(m), m);  // row_bcast15: rows 1, 3 absorb the row before
-    m = seq_compose(seq_dpp<0x143, 0xc>(m), m);  // row_bcast31: rows 2, 3 absorb rows 0-1
+    m = seq_wave_inclusive(m);
     if (lane == 63 && wave < NW) s_w[wave] = m;
     const SeqMap ex = seq_dpp<0x138, 0xf>(m);  // wave_shr:1: exclusive inside the wave, lane 0 reads the identity
     __syncthreads();
@@ -579,10 +600,19 @@ __device__ __forceinline__ SeqMap seq_block_before(SeqMap m, SeqMap *s_w, SeqMap
     static_assert(NW <= 16, "the waves' totals must fit one row of lanes");
     SeqMap v = seq_identity();
     if (lane < NW) v = s_w[lane];
-    v = seq_compose(seq_dpp<0x111, 0xf>(v), v);  // row_shr:1
-    v = seq_compose(seq_dpp<0x112, 0xf>(v), v);  // row_shr:2
-    if (NW > 4) v = seq_compose(seq_dpp<0x114, 0xf>(v), v);  // row_shr:4
-    if (NW > 8) v = seq_compose(seq_dpp<0x118, 0xf>(v), v);  // row_shr:8
+    if (__ballot(v.d0 != v.d1) == 0ull) {  // plain increments (see seq_wave_inclusive): at most 16 x 2^25
+        int sum = (int)v.d0;
+        sum += __builtin_amdgcn_update_dpp(0, sum, 0x111, 0xf, 0xf, true);  // row_shr:1
+        sum += __builtin_amdgcn_update_dpp(0, sum, 0x112, 0xf, 0xf, true);  // row_shr:2
+        if (NW > 4) sum += __builtin_amdgcn_update_dpp(0, sum, 0x114, 0xf, 0xf, true);  // row_shr:4
+        if (NW > 8) sum += __builtin_amdgcn_update_dpp(0, sum, 0x118, 0xf, 0xf, true);  // row_shr:8
+        v.d0 = v.d1 = seq_min_u32((uint32_t)sum, SEQ_SAT);
+    } else {
+        v = seq_compose(seq_dpp<0x111, 0xf>(v), v);  // row_shr:1
+        v = seq_compose(seq_dpp<0x112, 0xf>(v), v);  // row_shr:2
+        if (NW > 4) v = seq_compose(seq_dpp<0x114, 0xf>(v), v);  // row_shr:4
+        if (NW > 8) v = seq_compose(seq_dpp<0x118, 0xf>(v), v);  // row_shr:8
+    }
     const int w_uni = __builtin_amdgcn_readfirstlane(wave);
     SeqMap pre = seq_identity(), tot;
     tot.d0 = (uint32_t)__builtin_amdgcn_readlane((int)v.d0, NW - 1);
@@ -727,13 +757,7 @@ __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x
         if (t >= done) m = seq_map16(a, es, seq_ulp_scale(es < 26u ? 26u : es));
         if (t == 0) *s_first = 0xffffffffu;
         // inclusive scan of the wave, the waves' totals through LDS
-        SeqMap inc = m;
-        inc = seq_compose(seq_dpp<0x111, 0xf>(inc), inc);  // row_shr:1
-        inc = seq_compose(seq_dpp<0x112, 0xf>(inc), inc);  // row_shr:2
-        inc = seq_compose(seq_dpp<0x114, 0xf>(inc), inc);  // row_shr:4
-        inc = seq_compose(seq_dpp<0x118, 0xf>(inc), inc);  // row_shr:8
-        inc = seq_compose(seq_dpp<0x142, 0xa>(inc), inc);  // row_bcast15
-        inc = seq_compose(seq_dpp<0x143, 0xc>(inc), inc);  // row_bcast31
+        const SeqMap inc = seq_wave_inclusive(m);
         if (lane == 63) s_w[wave] = inc;
         const SeqMap ex = seq_dpp<0x138, 0xf>(inc);  // wave_shr:1: exclusive inside the wave
         __syncthreads();  // (1)

@@ -40,6 +40,9 @@ struct rbn_ctx {
     unsigned *dev_flags = nullptr;
     // the window-end kernel of the exact sums has been given its dynamic-LDS limit on this device
     bool seq_scan_prepared = false;
+    // the size (in blocks of the exact sums) of the last tensor summed and the windows its sums took
+    uint64_t seq_seen_blocks = 0;
+    int seq_seen_windows = 0;
 };
 
 constexpr int RBN_SPLITK_TILES = 16384;  // 64 MiB

@@ -248,6 +248,8 @@ struct SeqState {
     uint32_t rate_lo;   // multi: the cautious growth of S per block (f32 bits) behind the blocks' exponents
     uint32_t thr_bits;  // a sum queued behind another one: its mask threshold (f32 bits), set on the device
     uint64_t survivors;  // packing sums only: elements above the threshold, set by the window that ends the sum
+    uint32_t windows;   // windows folded so far (the host sizes the next sum's first batch by it)
+    uint32_t pad;
 };
 
 // A SeqMap from another lane by a DPP move: lanes without a source (and rows outside the
@@ -527,7 +529,7 @@ __global__ __launch_bounds__(kBlock) void seq_init_kernel(SeqState *__restrict__
     if (threadIdx.x == 0) {
         SeqState z;
         z.s_bits = 0, z.win = win0, z.pos = 0, z.done = 0, z.error = 0, z.saw_nan = 0, z.multi = 0;
-        z.fresh_from = 0, z.rate_lo = 0, z.thr_bits = 0, z.survivors = 0;
+        z.fresh_from = 0, z.rate_lo = 0, z.thr_bits = 0, z.survivors = 0, z.windows = 0, z.pad = 0;
         *state = z;
     }
 }
@@ -549,7 +551,7 @@ __global__ __launch_bounds__(kBlock) void seq_chain_init_kernel(const SeqState *
         const bool complete = p.done && !p.error && p.pos >= total_blocks && ((p.s_bits >> 23) & 0xffu) != 0xffu;
         SeqState z;
         z.s_bits = 0, z.win = 1u, z.pos = 0, z.done = complete ? 0u : 1u, z.error = complete ? 0u : 2u;
-        z.saw_nan = 0, z.multi = 0, z.fresh_from = 0, z.rate_lo = 0, z.survivors = 0;
+        z.saw_nan = 0, z.multi = 0, z.fresh_from = 0, z.rate_lo = 0, z.survivors = 0, z.windows = 0, z.pad = 0;
         const float mean = __uint_as_float(p.s_bits) / (float)n;
         z.thr_bits = __float_as_uint(mean * 0.7f);
         *state = z;
@@ -910,6 +912,8 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
         next.rate_lo = seq_multi_rate_lo(rate);
         next.saw_nan = 0;
         next.thr_bits = st0.thr_bits;
+        next.windows = st0.windows + 1u;
+        next.pad = 0;
         next.survivors = survivors_total;
         const uint64_t seen = pos0 + nblocks, before = st0.fresh_from;
         next.fresh_from = seen > before ? seen : before;
@@ -1338,6 +1342,13 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     // pair of launches returns at once: 4 us; another look by the host costs 10-25 us)
     int batch = 4;
     for (uint64_t b = total_blocks / SEQ_MULTI_LIMIT; b > 1; b >>= 1) ++batch;
+    // ... unless the context has just summed a tensor of this size: sums that stall (rounding eats the
+    // terms in the highest binades) and windows sized by a good rate need fewer, and a pair of
+    // launches that finds the sum complete still costs 6 us.  One spare beyond what the last
+    // sums of this size took; a sum that needs more costs a look by the host.
+    if (ctx->seq_seen_blocks == total_blocks && ctx->seq_seen_windows > 0 && ctx->seq_seen_windows + 1 < batch)
+        batch = ctx->seq_seen_windows + 1;
+    int windows_taken = 0;
     queue_batch(main_run, batch, true);
     SeqRun next_run{};
     if (follower) {
@@ -1352,6 +1363,7 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
     RBN_HIP(hipStreamSynchronize(ctx->stream));
     RBN_CHECK(run_to_end(main_run));
     SeqState *h_state = main_run.h_state;
+    windows_taken = (int)h_state->windows;
     const uint32_t s_bits = h_state->s_bits;
     const uint64_t pos = h_state->pos;
     float s;
@@ -1396,8 +1408,11 @@ int strict_abs_sum(rbn_ctx *ctx, const float *d_x, uint64_t n, int use_mask, flo
             else
                 *follower->h_survivors = h_next->survivors;
             follower->ran = true;
+            if ((int)h_next->windows > windows_taken) windows_taken = (int)h_next->windows;
         }
     }
+    ctx->seq_seen_blocks = total_blocks;
+    ctx->seq_seen_windows = windows_taken;
     return RBN_OK;
 }
 

@@ -819,6 +819,108 @@ __device__ __forceinline__ uint32_t seq_replay_block(const float *__restrict__ x
     return result_bits;
 }
 
+// The usual case of a crossing block, resolved with two barriers instead of five: S leaves its binade
+// once inside the block and ends one binade up.  The four working waves map their quarter of the
+// block for BOTH exponents at once (a map does not depend on the state, only on the exponent), so
+// that after one exchange of the quarters' maps the wave that holds the crossing can finish alone:
+// it finds the crossing chunk among its lanes, lets that lane add its sixteen terms, composes the
+// maps of its remaining lanes for the new exponent and walks through the quarters behind it.
+// Returns false (the same in every thread, nothing but LDS scratch touched) when the block is not
+// of that kind - a second crossing, a jump over a binade, an overflow: seq_replay_block then does
+// it in general.  Results as there: *s_bits_now, s_cross[0..1], valid after the last barrier inside.
+__device__ __forceinline__ bool seq_replay_block_once(const float *__restrict__ x, uint64_t n, uint64_t block_base,
+                                                      int use_mask, float thr, uint32_t es, uint32_t k_cur,
+                                                      SeqMap *s_w /* 8 slots */, uint32_t *s_bits_now,
+                                                      uint32_t *s_cross, unsigned *s_ok) {
+    if (es < 26u || es + 1u > 253u) return false;  // (uniform: below 26 terms are split in integer arithmetic)
+    const uint32_t t = threadIdx.x;
+    constexpr int NW = kBlock / 64;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(t >> 6));
+    if (wave >= NW) {
+        __syncthreads();  // (A) the quarters' maps
+        __syncthreads();  // (B) the result
+        return *s_ok != 0u;
+    }
+    const uint64_t base = block_base + (uint64_t)t * 16;
+    float a[16];
+    if (base + 16 <= n && (reinterpret_cast<uintptr_t>(x + base) & 15u) == 0) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float4 v = reinterpret_cast<const float4 *>(x + base)[j];
+            a[4 * j] = fabsf(v.x), a[4 * j + 1] = fabsf(v.y), a[4 * j + 2] = fabsf(v.z), a[4 * j + 3] = fabsf(v.w);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) a[i] = 0.0f;
+        for (int i = 0; i < 16; ++i) {
+            const uint64_t idx = base + i;
+            if (idx < n) a[i] = fabsf(x[idx]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a[i] = (!use_mask || a[i] > thr) ? a[i] : 0.0f;
+    const SeqMap m0 = seq_map16(a, es, seq_ulp_scale(es));
+    const SeqMap m1 = seq_map16(a, es + 1u, seq_ulp_scale(es + 1u));
+    const SeqMap inc0 = seq_wave_inclusive(m0);
+    const int lane = t & 63;
+    // the quarter's map for the new exponent: lane 63 of the scan of all its lanes
+    const SeqMap inc1 = seq_wave_inclusive(m1);
+    if (lane == 63) {
+        s_w[wave] = inc0;
+        s_w[NW + wave] = inc1;
+    }
+    if (t == 0) *s_ok = 0u;
+    __syncthreads();  // (A)
+    // the quarter in which k reaches 2^24, and the k that enters it (the same in every thread)
+    int q = -1;
+    uint32_t kq = k_cur, k = k_cur;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) {
+        const uint32_t k2 = seq_apply(s_w[w], k);
+        if (q < 0 && k2 >= SEQ_K_LIMIT) q = w, kq = k;
+        if (q < 0) k = k2;
+    }
+    if (wave == q) {
+        const SeqMap ex0 = seq_dpp<0x138, 0xf>(inc0);  // wave_shr:1: what lies before the lane, lane 0 the identity
+        const uint32_t kl = seq_apply(ex0, kq);
+        const bool crosses = kl < SEQ_K_LIMIT && seq_apply(m0, kl) >= SEQ_K_LIMIT;
+        const unsigned long long where = __ballot(crosses);
+        bool ok = where != 0ull;
+        const int tstar = ok ? __builtin_ctzll(where) : 0;
+        // the crossing chunk, replayed by its lane with ordinary f32 additions
+        float sum = __uint_as_float(seq_state_join(es, kl));
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sum = sum + a[i];
+        const uint32_t bits = (uint32_t)__builtin_amdgcn_readlane((int)__float_as_uint(sum), tstar);
+        uint32_t es2, k2;
+        seq_state_split(bits, &es2, &k2);
+        ok = ok && ((bits >> 23) & 0xffu) != 0xffu && es2 == es + 1u;
+        // the lanes behind it, for the new exponent
+        SeqMap rest = lane > tstar ? m1 : seq_identity();
+        rest = seq_wave_inclusive(rest);
+        SeqMap tail;
+        tail.d0 = (uint32_t)__builtin_amdgcn_readlane((int)rest.d0, 63);
+        tail.d1 = (uint32_t)__builtin_amdgcn_readlane((int)rest.d1, 63);
+        uint32_t k3 = seq_apply(tail, k2);
+        ok = ok && k3 < SEQ_K_LIMIT;
+        // and the quarters behind this one
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            if (w > q && ok) {
+                k3 = seq_apply(s_w[NW + w], k3);
+                ok = k3 < SEQ_K_LIMIT;
+            }
+        }
+        if (lane == 0 && ok) {
+            *s_bits_now = seq_state_join(es + 1u, k3);
+            s_cross[0] = bits, s_cross[1] = (uint32_t)q * 64u + (uint32_t)tstar + 1u;
+            *s_ok = 1u;
+        }
+    }
+    __syncthreads();  // (B)
+    return *s_ok != 0u;
+}
+
 // One workgroup of 1024 threads ends a window.
 // (1) Scan: walks the block maps of the window from the true state and finds the first
 //     block in which k reaches 2^24.
@@ -850,6 +952,7 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     __shared__ unsigned s_cnt0;
     __shared__ __attribute__((aligned(16))) float s_head[512];
     __shared__ uint32_t s_cross[2];
+    __shared__ unsigned s_once;
     const uint32_t t = threadIdx.x;
     // Windows of up to 1024 blocks (most of them) have one map per thread: it is requested
     // here, before the state is known, so that the two round trips overlap (the buffer holds
@@ -1031,8 +1134,12 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
                 break;  // the window is through, or the next block's pair does not hold es
             }
             const uint32_t cb = (uint32_t)(first_cross >> 32), k_cb = (uint32_t)first_cross;
-            (void)seq_replay_block(x, n, first + (uint64_t)cb * kSeqTile, use_mask, thr, es, k_cb, s_w, &s_first,
-                                   &s_bits_now, s_head, s_cross);
+            if (!seq_replay_block_once(x, n, first + (uint64_t)cb * kSeqTile, use_mask, thr, es, k_cb, s_w, &s_bits_now,
+                                       s_cross, &s_once)) {
+                __syncthreads();  // (s_once was read)
+                (void)seq_replay_block(x, n, first + (uint64_t)cb * kSeqTile, use_mask, thr, es, k_cb, s_w, &s_first,
+                                       &s_bits_now, s_head, s_cross);
+            }
             __syncthreads();  // the result is in LDS; s_w and s_min64 are rewritten in the next turn
             cur_bits = s_bits_now;
             cross_bits = s_cross[0], cross_chunks = s_cross[1], cross_block = cb, crossed = true;
@@ -1141,8 +1248,15 @@ __global__ __launch_bounds__(1024) void seq_scan_replay_kernel(
     }
 
     // ---- (2) replay of block cb
-    const uint32_t result_bits = seq_replay_block(x, n, first + (uint64_t)cb * kSeqTile, use_mask, thr, es, k_cur,
-                                                  s_w, &s_first, &s_bits_now, s_head, s_cross);
+    uint32_t result_bits;
+    if (seq_replay_block_once(x, n, first + (uint64_t)cb * kSeqTile, use_mask, thr, es, k_cur, s_w, &s_bits_now, s_cross,
+                              &s_once)) {
+        result_bits = s_bits_now;
+    } else {
+        __syncthreads();  // (s_once was read)
+        result_bits = seq_replay_block(x, n, first + (uint64_t)cb * kSeqTile, use_mask, thr, es, k_cur, s_w, &s_first,
+                                       &s_bits_now, s_head, s_cross);
+    }
     count_survivors(cb + 1);
     if (t == 0) finish(result_bits, cb + 1, s_cross[0], (double)((uint32_t)kBlock - s_cross[1]) / kBlock);
 }

@@ -137,6 +137,82 @@ ScanResult scan_stretch(const std::vector<SeqMap> &all_maps, uint32_t from, uint
 }
 }  // namespace
 
+// Counters of the two-barrier replay below: blocks it was tried on, blocks it resolved, and blocks
+// where its result differed from the general replay's (must stay 0).
+static uint64_t g_once_tried = 0, g_once_used = 0, g_once_differs = 0;
+extern "C" void seqsum_once_stats(uint64_t *tried, uint64_t *used, uint64_t *differs) {
+    *tried = g_once_tried, *used = g_once_used, *differs = g_once_differs;
+}
+
+// The usual crossing block as the device resolves it with two barriers: the quarters' maps for the
+// state's exponent and the next one, the quarter and then the chunk in which k reaches 2^24, that
+// chunk replayed, the chunks behind it and the quarters behind them for the new exponent.  Returns
+// false when the block is not of that kind.
+static bool replay_block_once(const float *x, uint64_t n, uint64_t bbase, int use_mask, float thr, uint32_t es,
+                              uint32_t k_cur, uint32_t *result_bits, uint32_t *cross_bits, uint32_t *cross_chunks) {
+    if (es < 26u || es + 1u > 253u) return false;
+    SeqMap m0[256], m1[256], q0[4], q1[4];
+    for (int t = 0; t < 256; ++t) {
+        m0[t] = thread_map(x, bbase + (uint64_t)t * 16, n, es, use_mask, thr);
+        m1[t] = thread_map(x, bbase + (uint64_t)t * 16, n, es + 1u, use_mask, thr);
+    }
+    for (int w = 0; w < 4; ++w) {
+        q0[w] = q1[w] = seq_identity();
+        for (int l = 0; l < 64; ++l) {
+            q0[w] = seq_compose(q0[w], m0[w * 64 + l]);
+            q1[w] = seq_compose(q1[w], m1[w * 64 + l]);
+        }
+    }
+    int q = -1;
+    uint32_t kq = k_cur, k = k_cur;
+    for (int w = 0; w < 4; ++w) {
+        const uint32_t k2 = seq_apply(q0[w], k);
+        if (q < 0 && k2 >= SEQ_K_LIMIT) q = w, kq = k;
+        if (q < 0) k = k2;
+    }
+    if (q < 0) return false;
+    int tstar = -1;
+    uint32_t kl = kq;
+    for (int l = 0; l < 64; ++l) {
+        if (kl < SEQ_K_LIMIT && seq_apply(m0[q * 64 + l], kl) >= SEQ_K_LIMIT) {
+            tstar = l;
+            break;
+        }
+        kl = seq_apply(m0[q * 64 + l], kl);
+    }
+    if (tstar < 0) return false;
+    const uint32_t jb = seq_state_join(es, kl);
+    float s;
+    std::memcpy(&s, &jb, 4);
+    for (int i = 0; i < 16; ++i) {
+        const uint64_t idx = bbase + (uint64_t)(q * 64 + tstar) * 16 + i;
+        float av = 0.0f;
+        bool take = false;
+        if (idx < n) {
+            av = std::fabs(x[idx]);
+            take = use_mask ? (av > thr) : true;
+        }
+        volatile float t2 = s + (take ? av : 0.0f);
+        s = t2;
+    }
+    uint32_t bits;
+    std::memcpy(&bits, &s, 4);
+    uint32_t es2, k2;
+    seq_state_split(bits, &es2, &k2);
+    if (((bits >> 23) & 0xffu) == 0xffu || es2 != es + 1u) return false;
+    SeqMap tail = seq_identity();
+    for (int l = tstar + 1; l < 64; ++l) tail = seq_compose(tail, m1[q * 64 + l]);
+    uint32_t k3 = seq_apply(tail, k2);
+    if (k3 >= SEQ_K_LIMIT) return false;
+    for (int w = q + 1; w < 4; ++w) {
+        k3 = seq_apply(q1[w], k3);
+        if (k3 >= SEQ_K_LIMIT) return false;
+    }
+    *result_bits = seq_state_join(es + 1u, k3);
+    *cross_bits = bits, *cross_chunks = (uint32_t)(q * 64 + tstar + 1);
+    return true;
+}
+
 // The replay of one block (the second half of the window-end kernel): crossings inside the
 // block are resolved one after another.  Returns the state after the block as f32 bits.
 static uint32_t replay_block(const float *x, uint64_t n, uint64_t bbase, int use_mask, float thr,
@@ -260,6 +336,16 @@ extern "C" float seqsum_host(const float *x, uint64_t n, int use_mask, float thr
             }
             cur_bits = replay_block(x, n, first + (b_cur + sr.cross_block) * kTile, use_mask, thr, es, sr.k,
                                     &cross_bits, &cross_chunks);
+            if (pos + b_cur + sr.cross_block > 0) {  // (the first block of a sum is always replayed in general)
+                uint32_t once_bits, once_cross, once_chunks;
+                ++g_once_tried;
+                if (replay_block_once(x, n, first + (b_cur + sr.cross_block) * kTile, use_mask, thr, es, sr.k,
+                                      &once_bits, &once_cross, &once_chunks)) {
+                    ++g_once_used;
+                    if (once_bits != cur_bits || once_cross != cross_bits || once_chunks != cross_chunks)
+                        ++g_once_differs;
+                }
+            }
             crossed = true, cross_block = b_cur + sr.cross_block;
             b_cur += (uint64_t)sr.cross_block + 1;
             if (((cur_bits >> 23) & 0xff) == 0xff || b_cur >= win) break;

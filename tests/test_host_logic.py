@@ -123,6 +123,8 @@ def seqsum(tmp_path_factory):
     L.seqsum_compare_block_forms.argtypes = [C.c_uint64, C.c_uint64, C.POINTER(C.c_uint64)]
     L.seqsum_compare_map16.restype = C.c_uint64
     L.seqsum_compare_map16.argtypes = [C.c_uint64, C.c_uint64, C.POINTER(C.c_uint64)]
+    L.seqsum_once_stats.restype = None
+    L.seqsum_once_stats.argtypes = [C.POINTER(C.c_uint64)] * 3
     L.seqsum_check_map_slots.restype = C.c_uint64
     L.seqsum_check_map_slots.argtypes = [C.c_uint32]
     return L
@@ -188,6 +190,22 @@ def test_a_window_longer_than_one_stretch_is_walked_stretch_by_stretch(seqsum):
     it = C.c_uint64()
     got = np.float32(seqsum.seqsum_host(x.ctypes.data, x.size, 0, 0.0, C.byref(it), None))
     assert got == np.float32(65536 + blocks) and it.value == 5
+
+
+def test_two_barrier_replay_agrees_with_the_general_one(seqsum):
+    # every crossing block that the short replay (one crossing, one binade up) resolves must come out as the
+    # general replay has it: state after the block, state behind the crossing chunk, chunks folded up to it
+    rng = np.random.default_rng(11)
+    for scale, n in ((0.02, 3_000_000), (1.0, 700_000), (1e-3, 2_000_000), (30.0, 400_001)):
+        x = (rng.standard_normal(n) * scale).astype(np.float32)
+        x[rng.integers(0, n, 50)] *= 1000.0          # a few terms that jump over binades
+        for mask, thr in ((0, 0.0), (1, float(np.median(np.abs(x))))):
+            got = np.float32(seqsum.seqsum_host(x.ctypes.data, n, mask, thr, None, None))
+            want = np.float32(seqsum.seqsum_literal(x.ctypes.data, n, mask, thr))
+            assert got.view(np.uint32) == want.view(np.uint32)
+    tried, used, differs = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    seqsum.seqsum_once_stats(C.byref(tried), C.byref(used), C.byref(differs))
+    assert differs.value == 0 and used.value > 20 and tried.value >= used.value
 
 
 def test_float_and_integer_term_splits_agree(seqsum):

@@ -47,8 +47,11 @@ __device__ __forceinline__ uint32_t ternary_code(float v, float threshold) {
 // ---------------------------------------------------------------------------
 template <bool NT>
 __global__ __launch_bounds__(kBlock) void pack_ternary_kernel(
-    const float *__restrict__ x, uint64_t n, float threshold, uint32_t *__restrict__ packed,
-    uint64_t n_tiles, unsigned long long *__restrict__ survivors, double *__restrict__ psum) {
+    const float *__restrict__ x, uint64_t n, float threshold_arg, const float *__restrict__ threshold_ptr,
+    uint32_t *__restrict__ packed, uint64_t n_tiles, unsigned long long *__restrict__ survivors,
+    double *__restrict__ psum) {
+    // (the tree-sum quantiser queues this pass behind its sum: the threshold then comes from the device)
+    const float threshold = threshold_ptr ? *threshold_ptr : threshold_arg;
     __shared__ unsigned s_cnt[kBlock / 64];
     __shared__ double s_sum[kBlock / 64];
     double acc = 0.0;  // sum of the survivors' |x| (tree mode: one partial per workgroup)
@@ -205,7 +208,9 @@ __global__ __launch_bounds__(kBlock) void abs_sum_tree_partial_kernel(
 
 __global__ __launch_bounds__(kBlock) void abs_sum_tree_final_kernel(
     const double *__restrict__ psum, const unsigned long long *__restrict__ pcnt, int nparts,
-    float *__restrict__ out_sum, unsigned long long *__restrict__ out_cnt) {
+    float *__restrict__ out_sum, unsigned long long *__restrict__ out_cnt,
+    uint64_t n = 0, float *__restrict__ out_threshold = nullptr /* (sum / n) * 0.7, quantization.rs:79 */,
+    unsigned long long *__restrict__ clear = nullptr /* the packing pass's survivor counter */) {
     __shared__ double s_sum[kBlock];
     __shared__ unsigned long long s_cnt[kBlock];
     double acc = 0.0;
@@ -225,8 +230,14 @@ __global__ __launch_bounds__(kBlock) void abs_sum_tree_final_kernel(
         __syncthreads();
     }
     if (threadIdx.x == 0) {
-        *out_sum = (float)s_sum[0];
+        const float sum = (float)s_sum[0];
+        *out_sum = sum;
         *out_cnt = s_cnt[0];
+        if (out_threshold) {
+            const float mean = sum / (float)n;
+            *out_threshold = mean * 0.7f;
+        }
+        if (clear) *clear = 0ull;
     }
 }
 
@@ -1346,8 +1357,10 @@ struct ReduceScratch {
     SeqState seq_next;  // the sum queued behind `seq`
     unsigned long long survivors;
     float tree_sum;
-    uint32_t pad0;
+    float tree_threshold;  // the tree-sum quantiser: the threshold its packing pass reads
     unsigned long long tree_cnt;
+    float pack_sum;  // ... and the survivors' sum of that pass
+    uint32_t pad0;
 };
 constexpr size_t kScratchHeader = 256;
 static_assert(sizeof(ReduceScratch) <= kScratchHeader, "scratch header too small");
@@ -1590,10 +1603,10 @@ int pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold, ui
     const unsigned grid = (unsigned)(tiles < (uint64_t)kPackGrid ? tiles : (uint64_t)kPackGrid);
     if (n * 4 > kStreamBytes)
         pack_ternary_kernel<true><<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
-            d_x, n, threshold, (uint32_t *)d_packed, tiles, d_cnt, d_psum);
+            d_x, n, threshold, nullptr, (uint32_t *)d_packed, tiles, d_cnt, d_psum);
     else
         pack_ternary_kernel<false><<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
-            d_x, n, threshold, (uint32_t *)d_packed, tiles, d_cnt, d_psum);
+            d_x, n, threshold, nullptr, (uint32_t *)d_packed, tiles, d_cnt, d_psum);
     if (d_psum)
         sum_partials_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(d_psum, (int)grid, &scr->tree_sum);
     RBN_HIP(hipGetLastError());
@@ -1605,6 +1618,55 @@ int pack_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, float threshold, ui
         if (h_survivors) memcpy(h_survivors, mb, 8);
         if (h_survivor_sum) memcpy(h_survivor_sum, mb + 8, 4);
     }
+    return RBN_OK;
+}
+
+// The tree-sum quantiser in one queue: sum, threshold on the device, packing pass with the
+// survivors' count and sum, one look by the host at the end.  *chained is false when the device's
+// threshold is not the host's own (sum / n) * 0.7 bit for bit: the caller then packs again the
+// ordinary way.
+int tree_quantize_chained(rbn_ctx *ctx, const float *d_x, uint64_t n, uint8_t *d_packed, float *h_sum,
+                          uint64_t *h_survivors, float *h_survivor_sum, bool *chained) {
+    *chained = false;
+    const uint64_t tiles = (n + kSeqTile - 1) / kSeqTile;
+    if (n == 0 || tiles > 0x7fffffffull) return RBN_OK;
+    void *ws = nullptr;
+    RBN_CHECK(rbn_workspace(ctx, kScratchHeader + kTreeParts * 16 + (size_t)kPackGrid * sizeof(double), &ws));
+    ReduceScratch *scr = (ReduceScratch *)ws;
+    double *psum = (double *)((char *)ws + kScratchHeader);
+    unsigned long long *pcnt = (unsigned long long *)(psum + kTreeParts);
+    double *pack_psum = (double *)((char *)ws + kScratchHeader + kTreeParts * 16);
+    const int parts = (int)(tiles < (uint64_t)kTreeParts ? tiles : (uint64_t)kTreeParts);
+    const unsigned grid = (unsigned)(tiles < (uint64_t)kPackGrid ? tiles : (uint64_t)kPackGrid);
+    const bool stream = n * 4 > kStreamBytes;
+    if (stream)
+        abs_sum_tree_partial_kernel<true><<<dim3(parts), dim3(kBlock), 0, ctx->stream>>>(d_x, n, 0, 0.0f, psum, pcnt);
+    else
+        abs_sum_tree_partial_kernel<false><<<dim3(parts), dim3(kBlock), 0, ctx->stream>>>(d_x, n, 0, 0.0f, psum, pcnt);
+    abs_sum_tree_final_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(
+        psum, pcnt, parts, &scr->tree_sum, &scr->tree_cnt, n, &scr->tree_threshold, &scr->survivors);
+    if (stream)
+        pack_ternary_kernel<true><<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
+            d_x, n, 0.0f, &scr->tree_threshold, (uint32_t *)d_packed, tiles, &scr->survivors, pack_psum);
+    else
+        pack_ternary_kernel<false><<<dim3(grid), dim3(kBlock), 0, ctx->stream>>>(
+            d_x, n, 0.0f, &scr->tree_threshold, (uint32_t *)d_packed, tiles, &scr->survivors, pack_psum);
+    sum_partials_kernel<<<dim3(1), dim3(kBlock), 0, ctx->stream>>>(pack_psum, (int)grid, &scr->pack_sum);
+    RBN_HIP(hipGetLastError());
+    char *mb = (char *)ctx->mailbox;
+    constexpr size_t kBack = offsetof(ReduceScratch, pad0) - offsetof(ReduceScratch, survivors);  // survivors .. pack_sum
+    RBN_HIP(hipMemcpyAsync(mb, &scr->survivors, kBack, hipMemcpyDeviceToHost, ctx->stream));
+    RBN_HIP(hipStreamSynchronize(ctx->stream));
+    ReduceScratch back;
+    memcpy(&back.survivors, mb, kBack);
+    *h_sum = back.tree_sum;
+    volatile float mean = back.tree_sum / (float)n;
+    volatile float want = mean * 0.7f;
+    float want_f = want;
+    if (memcmp(&want_f, &back.tree_threshold, 4) != 0) return RBN_OK;
+    *h_survivors = back.survivors;
+    *h_survivor_sum = back.pack_sum;
+    *chained = true;
     return RBN_OK;
 }
 
@@ -1658,9 +1720,13 @@ int rbn_quantize_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, int mode, u
     }
     // quantization.rs:79: (sum / n as f32) * 0.7
     float sum = 0.0f;
-    if (mode == RBN_SUM_TREE) RBN_CHECK(tree_abs_sum(ctx, d_x, n, 0, 0.0f, &sum, nullptr));
     uint64_t survivors = 0;
     float nz_sum = 0.0f;
+    bool tree_chained = false;
+    if (mode == RBN_SUM_TREE) {
+        RBN_CHECK(tree_quantize_chained(ctx, d_x, n, d_packed, &sum, &survivors, &nz_sum, &tree_chained));
+        if (!tree_chained) RBN_CHECK(tree_abs_sum(ctx, d_x, n, 0, 0.0f, &sum, nullptr));
+    }
     SeqFollower masked{d_packed, &nz_sum, &survivors, false};
     if (mode != RBN_SUM_TREE)
         RBN_CHECK(strict_abs_sum(ctx, d_x, n, 0, 0.0f, &sum, nullptr, nullptr, &masked));
@@ -1668,9 +1734,9 @@ int rbn_quantize_ternary(rbn_ctx *ctx, const float *d_x, uint64_t n, int mode, u
     volatile float threshold = mean * 0.7f;
     // quantization.rs:100 (pack) and the survivor count of :82-91
     // (one pass in either mode: the survivors' sum, their count and the packed words)
-    if (mode == RBN_SUM_TREE)
-        RBN_CHECK(pack_ternary(ctx, d_x, n, threshold, d_packed, &survivors, &nz_sum));
-    else if (!masked.ran)
+    if (mode == RBN_SUM_TREE) {
+        if (!tree_chained) RBN_CHECK(pack_ternary(ctx, d_x, n, threshold, d_packed, &survivors, &nz_sum));
+    } else if (!masked.ran)
         RBN_CHECK(strict_abs_sum(ctx, d_x, n, 1, threshold, &nz_sum, d_packed, &survivors));
     // quantization.rs:93-97
     float scale = 1.0f;

@@ -235,6 +235,24 @@ def test_quantize_tree_mode_is_close_but_flagged(ctx):
     assert (packed == O.pack_ternary_bits(w, thr)).all()
 
 
+@pytest.mark.parametrize("n", [1, 17, 4097, 70_001, 3_000_000, 60_000_000])
+def test_quantize_tree_mode_threshold_from_the_device(ctx, n):
+    """The tree-sum quantiser queues its packing pass behind the sum and takes the threshold from the
+    device: threshold = (sum / n) * 0.7 of the sum it returns, bit for bit; count and packed codes are
+    those of that threshold; the survivors' mean is their f64 mean."""
+    w = synth_normal(40 + n % 97, 0.05, (n,))
+    d_x = ctx.to_device(w)
+    tree_sum, _ = ctx.abs_sum(d_x, n, TREE)
+    _, packed, scale, thr, cnt = device_quantize(ctx, w, TREE)
+    assert bits(thr) == bits(np.float32(np.float32(tree_sum) / np.float32(n)) * np.float32(0.7))
+    assert abs(float(tree_sum) - np.abs(w).astype(np.float64).sum()) <= 1e-6 * max(1.0, float(tree_sum))
+    keep = np.abs(w) > thr
+    assert cnt == int(keep.sum())
+    if cnt:
+        assert abs(float(scale) - np.abs(w)[keep].astype(np.float64).mean()) < 1e-6
+    assert (packed == O.pack_ternary_bits(w, thr)).all()
+
+
 def test_quantize_edge_tensors(ctx):
     for x in (np.zeros(10, dtype=np.float32), np.full(37, 3.0, dtype=np.float32),
               np.array([np.nan, 1.0, -2.0, 0.25], dtype=np.float32)):
